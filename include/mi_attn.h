@@ -1,0 +1,252 @@
+/*
+ * mi_attn.h - C ABI of the MI355X (gfx950) attention forward library.
+ *
+ * The upstream project (rookie-joe/TritonOps) has no FFI of its own: its
+ * boundary is a set of Python launchers that hand torch tensors to Triton
+ * kernels.  Every entry point below replaces one such launcher + kernel pair;
+ * the citation names the reference interface it stands in for (paths relative
+ * to the reference checkout).
+ *
+ * Conventions shared by all entry points
+ *   - plain C structs of pointers, element strides and sizes; no torch types;
+ *   - every struct starts with `struct_size` (sizeof the struct as the caller
+ *     compiled it) so the library can reject a mismatched caller;
+ *   - device pointers are raw HIP device addresses, `stream` is a hipStream_t
+ *     passed as void* (NULL = the null stream);
+ *   - the innermost (head_dim) axis of q/k/v/o must be contiguous and every
+ *     row must start on a 16-byte boundary (strides are in ELEMENTS);
+ *   - return value: MI_OK (0) or a negative mi_status; nothing throws, nothing
+ *     allocates or frees device memory, nothing synchronises the device;
+ *   - all argument validation happens on the host before any HIP call, so it
+ *     can be exercised on a machine without a GPU;
+ *   - log-sum-exp values are base 2 of the scaled scores, fp32:
+ *       lse2 = log2( sum_j 2^(q.k_j * scale_log2) ),  scale_log2 = scale*log2(e)
+ *     exactly as flash_attn_triton/flash_attn_triton.py:163,170,180,839;
+ *   - q-head h reads kv-head h / (heads_q / heads_kv)
+ *     (flash_attn_triton/flash_attn_triton.py:86-87,616).
+ */
+#ifndef MI_ATTN_H
+#define MI_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI_ATTN_ABI_VERSION 1
+
+/* KV tile edge (tokens) of the prefill kernels and block edge of the block
+ * sparse layouts; fixed at build time. */
+#define MI_ATTN_BLOCK 64
+
+typedef enum mi_dtype {
+  MI_DTYPE_BF16 = 0,
+  MI_DTYPE_F16 = 1
+} mi_dtype;
+
+typedef enum mi_status {
+  MI_OK = 0,
+  MI_ERR_NULL_POINTER = -1,   /* a required pointer is NULL                    */
+  MI_ERR_STRUCT_SIZE = -2,    /* struct_size does not match this library       */
+  MI_ERR_DTYPE = -3,          /* dtype is not MI_DTYPE_BF16 / MI_DTYPE_F16     */
+  MI_ERR_HEAD_DIM = -4,       /* head_dim not in {64, 96, 128}                 */
+  MI_ERR_GQA = -5,            /* heads_q % heads_kv != 0 or a count <= 0       */
+  MI_ERR_SHAPE = -6,          /* negative / zero / overflowing extent          */
+  MI_ERR_STRIDE = -7,         /* stride not a multiple of 8 elements (16 B)    */
+  MI_ERR_ALIGNMENT = -8,      /* base pointer not 16-byte aligned              */
+  MI_ERR_SCALE = -9,          /* scale_log2 not finite or <= 0                 */
+  MI_ERR_WORKSPACE = -10,     /* workspace too small / splits out of range     */
+  MI_ERR_SPARSE_LAYOUT = -11, /* block size / index list arguments invalid     */
+  MI_ERR_LAUNCH = -12,        /* hipLaunchKernel reported an error             */
+  MI_ERR_NO_DEVICE = -13      /* no HIP device / wrong architecture            */
+} mi_status;
+
+/* ------------------------------------------------------------------------- */
+/* Dense forward.
+ * Replaces flash_attn_triton_fwd + flash_attn_fwd_kernel
+ * (flash_attn_triton/flash_attn_triton.py:595-658, :52-180) for the packed
+ * var-len causal GQA form, and the [B,H,N,D] kernels of
+ * tutorial/4.3.multi_head_attention.py:45-194 (non-causal) and
+ * tutorial/4.4.causal_attention.py:133-180 (causal) for the batched form.
+ *
+ * Two addressing modes, one kernel:
+ *   cu_seqlens != NULL : packed. Token t of sequence b lives at row
+ *                        cu_seqlens[b]+t; *_stride_b is ignored.
+ *   cu_seqlens == NULL : batched. Every sequence has max_seqlen tokens and
+ *                        sequence b starts at b * *_stride_b.
+ * Rows whose sequence has length 0 are never written.
+ */
+typedef struct mi_attn_fwd_args {
+  uint32_t struct_size;
+  int32_t dtype;                 /* mi_dtype of q, k, v, o                     */
+  const void *q, *k, *v;         /* device                                     */
+  void *o;                       /* device, dtype as q                         */
+  float *lse;                    /* device, fp32 base-2 LSE; may be NULL       */
+  int64_t q_stride_b, q_stride_s, q_stride_h;
+  int64_t k_stride_b, k_stride_s, k_stride_h;
+  int64_t v_stride_b, v_stride_s, v_stride_h;
+  int64_t o_stride_b, o_stride_s, o_stride_h;
+  int64_t lse_stride_b, lse_stride_s, lse_stride_h;
+  const int32_t *cu_seqlens;     /* device [batch+1] or NULL                   */
+  int32_t batch, heads_q, heads_kv;
+  int32_t max_seqlen;            /* upper bound of every sequence length       */
+  int32_t head_dim;              /* 64, 96 or 128 (q, k and v alike)           */
+  int32_t causal;                /* 0 / 1                                      */
+  float scale_log2;              /* softmax scale * log2(e), > 0               */
+} mi_attn_fwd_args;
+
+int mi_attn_fwd(const mi_attn_fwd_args *args, void *stream);
+
+/* ------------------------------------------------------------------------- */
+/* Block-sparse forward (always token-causal).
+ * Replaces the sparse launcher + kernel of
+ * flash_attn_triton/flash_attn_sparse_attn_triton.py:237-326, :47-234, whose
+ * mask (oracle :422-433) is  k <= q  and  (q < k + local_window or
+ * k < global_window); generalised to an arbitrary list of live 64x64 blocks.
+ *
+ * Layout: CSR over query blocks of MI_ATTN_BLOCK tokens (block coordinates are
+ * relative to each sequence's first token).  Query block i of (batch b, head
+ * h) walks  col_idx[ off + row_ptr[i] .. off + row_ptr[i+1] )  with
+ *   row_ptr taken at   row_ptr + b*row_ptr_stride_b + h*row_ptr_stride_h
+ *   col_idx taken at   col_idx + b*col_idx_stride_b + h*col_idx_stride_h
+ * (strides of 0 broadcast one mask over batch and/or heads).  Column indices
+ * must be ascending, unique and <= i.  Inside a live block, keys beyond the
+ * query (causal) or beyond the sequence are masked per token.
+ *
+ * window_local / window_global: when window_local >= 0 the reference's token
+ * window is applied on top of the block list inside every live block:
+ *   allowed(q,k) = k <= q and (q - k < window_local or k < window_global).
+ * Pass -1 / -1 for a pure block mask.
+ * A query row with no allowed key yields o = 0 and lse = -inf.
+ */
+typedef struct mi_attn_sparse_args {
+  uint32_t struct_size;
+  int32_t dtype;
+  const void *q, *k, *v;
+  void *o;
+  float *lse;                    /* may be NULL                                */
+  int64_t q_stride_b, q_stride_s, q_stride_h;
+  int64_t k_stride_b, k_stride_s, k_stride_h;
+  int64_t v_stride_b, v_stride_s, v_stride_h;
+  int64_t o_stride_b, o_stride_s, o_stride_h;
+  int64_t lse_stride_b, lse_stride_s, lse_stride_h;
+  const int32_t *cu_seqlens;     /* device [batch+1] or NULL (batched)         */
+  const int32_t *row_ptr;        /* device [n_q_blocks+1] per (b,h) slice      */
+  const int32_t *col_idx;        /* device                                     */
+  int64_t row_ptr_stride_b, row_ptr_stride_h;
+  int64_t col_idx_stride_b, col_idx_stride_h;
+  int32_t batch, heads_q, heads_kv;
+  int32_t max_seqlen;
+  int32_t head_dim;
+  int32_t block_size;            /* must equal MI_ATTN_BLOCK                   */
+  int32_t window_local;          /* tokens, or -1                              */
+  int32_t window_global;         /* tokens, or -1                              */
+  float scale_log2;
+} mi_attn_sparse_args;
+
+int mi_attn_fwd_blocksparse(const mi_attn_sparse_args *args, void *stream);
+
+/* ------------------------------------------------------------------------- */
+/* Single-query decoding, dense and block-sparse.
+ * Replaces flash_attention_decoding (flash_attn_triton/flash_attn_decoding.py
+ * :213-336: pass 1 kernel :9-122, merge kernel :126-210) and
+ * flash_attention_sparse_decoding (flash_attn_triton/
+ * flash_attn_decoding_sparse.py:222-365: pass 1 :10-127, merge :131-219).
+ *
+ * q [batch, heads_q, head_dim]; k, v padded per sequence: token t of sequence
+ * b, kv-head h at  b*stride_b + t*stride_s + h*stride_h ; only the first
+ * seq_lens[b] tokens are read (flash_attn_decoding.py:46-48,80).  The G =
+ * heads_q/heads_kv query heads of one kv-head are processed together so every
+ * K/V byte is fetched from HBM once.
+ *
+ * Pass 1 splits each sequence into chunks of `split_tokens` tokens (dense) or
+ * `split_blocks` listed blocks (sparse); one workgroup per (chunk, kv-head,
+ * batch) writes an un-normalised fp32 partial output and its base-2 LSE into
+ * the workspace.  Pass 2 merges the partials (flash_attn_decoding.py:171-208).
+ * seq_lens[b] == 0 gives an all-zero output row (flash_attn_decoding.py:49-50,
+ * 151,197-210).
+ *
+ * Sparse form (block_idx != NULL): kv-head h of batch b reads the token blocks
+ *   block_idx[b*block_idx_stride_b + h*block_idx_stride_h + i],
+ *   i < (block_cnt ? block_cnt[b*heads_kv + h] : max_blocks),
+ * each `block_size` (64) tokens; indices must be unique and in range
+ * [0, ceil(seq_len/block_size)); tokens >= seq_len are masked.  On top of the
+ * list an optional token window reproduces flash_attn_decoding_sparse.py
+ * :391-396:  allowed(k) = k < window_global or k >= seq_len - window_local
+ * (pass -1/-1 to disable).
+ */
+typedef struct mi_decode_args {
+  uint32_t struct_size;
+  int32_t dtype;
+  const void *q, *k, *v;
+  void *o;                       /* [batch, heads_q, head_dim], dtype as q     */
+  float *lse;                    /* [batch, heads_q] fp32 base-2; may be NULL  */
+  int64_t q_stride_b, q_stride_h;
+  int64_t k_stride_b, k_stride_s, k_stride_h;
+  int64_t v_stride_b, v_stride_s, v_stride_h;
+  int64_t o_stride_b, o_stride_h;
+  const int32_t *seq_lens;       /* device [batch]; or                         */
+  const int32_t *cu_seqlens;     /* device [batch+1] (lengths = differences);  */
+                                 /* exactly one of the two is non-NULL         */
+  int32_t batch, heads_q, heads_kv;
+  int32_t max_seqlen;            /* upper bound of every length (grid size)    */
+  int32_t head_dim;              /* 64, 96 or 128                              */
+  float scale_log2;
+  /* split-KV */
+  int32_t split_tokens;          /* dense: tokens per workgroup, multiple of 64*/
+  void *workspace;               /* device, mi_decode_workspace_bytes() bytes  */
+  size_t workspace_bytes;
+  /* block-sparse (all ignored when block_idx == NULL) */
+  const int32_t *block_idx;      /* device                                     */
+  const int32_t *block_cnt;      /* device [batch*heads_kv] or NULL            */
+  int64_t block_idx_stride_b, block_idx_stride_h;
+  int32_t max_blocks;            /* list capacity per (b, kv-head)             */
+  int32_t block_size;            /* must equal MI_ATTN_BLOCK                   */
+  int32_t split_blocks;          /* sparse: listed blocks per workgroup        */
+  int32_t window_local;          /* tokens, or -1                              */
+  int32_t window_global;         /* tokens, or -1                              */
+} mi_decode_args;
+
+/* Number of pass-1 chunks per sequence for these arguments (host only). */
+int mi_decode_num_splits(const mi_decode_args *args);
+/* Bytes of workspace the two passes need: fp32 partial o + fp32 lse2. */
+size_t mi_decode_workspace_bytes(const mi_decode_args *args);
+/* Heuristic chunk length (tokens, multiple of 64) that fills `num_cus` compute
+ * units for the given problem; host only. */
+int mi_decode_choose_split_tokens(int batch, int heads_kv, int max_seqlen,
+                                  int num_cus);
+
+/* Pass 1 only: partials into the workspace. */
+int mi_decode_splitkv(const mi_decode_args *args, void *stream);
+/* Pass 2 only: merge the workspace into o (and lse). */
+int mi_decode_merge(const mi_decode_args *args, void *stream);
+/* Both passes back to back on `stream`. */
+int mi_decode(const mi_decode_args *args, void *stream);
+
+/* ------------------------------------------------------------------------- */
+/* Introspection (host only). */
+int mi_abi_version(void);
+/* Message of the last failing call on this thread ("" if none). */
+const char *mi_last_error(void);
+/* Name of a status code. */
+const char *mi_status_name(int status);
+/* Validate without launching (what the launch entry points run first). */
+int mi_attn_fwd_validate(const mi_attn_fwd_args *args);
+int mi_attn_fwd_blocksparse_validate(const mi_attn_sparse_args *args);
+int mi_decode_validate(const mi_decode_args *args);
+
+/* Average device time per launch, measured with HIP events on `stream` around
+ * `iters` back-to-back launches of the given entry point (after `warmup`
+ * untimed ones).  Blocks the calling thread; for benchmarking only.
+ * kind: 0 = mi_attn_fwd, 1 = mi_attn_fwd_blocksparse, 2 = mi_decode,
+ *       3 = mi_decode_splitkv, 4 = mi_decode_merge.
+ * Returns MI_OK and writes milliseconds to *ms_per_launch. */
+int mi_time_launches(int kind, const void *args, void *stream, int warmup,
+                     int iters, float *ms_per_launch);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI_ATTN_H */

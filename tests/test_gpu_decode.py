@@ -1,0 +1,139 @@
+"""GPU parity of the decoding kernels (dense / window / block-index) through
+the C ABI against the CPU oracle."""
+import pytest
+import torch
+
+from oracle import attention_oracle as orc
+from tests.util import LSE_TOL, TOL, assert_close, cu_from, randn
+
+pytestmark = pytest.mark.gpu
+
+
+def _kv(B, L, Hkv, D, dtype, seed):
+    return randn((B, L, Hkv, D), seed, dtype), randn((B, L, Hkv, D), seed + 1, dtype)
+
+
+# lengths of the reference's test (flash_attn_triton/flash_attn_decoding.py:383)
+# and its head_dim / dtype (D=96, fp16, :378-403), plus GQA and bf16 D=128
+@pytest.mark.parametrize("Hq,Hkv,D,dtype", [
+    (2, 2, 96, torch.float16),
+    (32, 8, 128, torch.bfloat16),
+    (8, 1, 64, torch.bfloat16),
+    (6, 2, 128, torch.float16),
+])
+def test_dense_decode_matches_oracle(Hq, Hkv, D, dtype):
+    import tritonops_amd as ta
+
+    lens = torch.tensor([512, 2049, 8192, 0, 1, 63, 64, 65], dtype=torch.int32)
+    B, L = len(lens), int(lens.max())
+    q = randn((B, Hq, D), 1, dtype)
+    k, v = _kv(B, L, Hkv, D, dtype, 2)
+    want, want_lse = orc.flash_attn_decoding_torch(q, k, v, lens, faithful=True, return_lse=True)
+    exact = orc.flash_attn_decoding_torch(q, k, v, lens, faithful=False)
+    cu = cu_from(lens)
+    got, lse = ta.flash_attention_decoding(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), return_lse=True)
+    assert got.shape == (B, Hq, D) and got.dtype == dtype
+    assert_close(got, exact, TOL, "o vs fp32 math")
+    assert_close(got, want, TOL, "o vs reference-dtype oracle")
+    assert torch.equal(got[3].cpu(), torch.zeros(Hq, D, dtype=dtype))       # len 0 -> zeros
+    assert_close(got[4], v[4, 0].repeat_interleave(Hq // Hkv, 0), 1e-6)     # len 1 -> v[0]
+    fin = torch.isfinite(want_lse)
+    assert torch.equal(torch.isfinite(lse.cpu()), fin)
+    assert (lse.cpu()[fin] - want_lse[fin]).abs().max() <= LSE_TOL
+    # split invariance: any chunking gives the same answer up to fp32 rounding
+    for st in (64, 256, 8192):
+        alt = ta.flash_attention_decoding(q.cuda(), k.cuda(), v.cuda(), None, seq_lens=lens.cuda(), split_tokens=st)
+        assert_close(alt, got, 4e-3, "split_tokens=%d" % st)
+
+
+def test_decode_on_transposed_cache_and_scale():
+    """KV memory [B,Hkv,L,D] passed as a [B,L,Hkv,D] view, explicit qk_scale."""
+    import tritonops_amd as ta
+
+    B, Hq, Hkv, L, D = 3, 16, 4, 1000, 128
+    lens = torch.tensor([1000, 333, 17], dtype=torch.int32)
+    q = randn((B, Hq, D), 4)
+    kc, vc = randn((B, Hkv, L, D), 5), randn((B, Hkv, L, D), 6)
+    k, v = kc.transpose(1, 2), vc.transpose(1, 2)
+    want = orc.flash_attn_decoding_torch(q, k, v, lens, qk_scale=0.05, faithful=False)
+    got = ta.flash_attention_decoding(q.cuda(), kc.cuda().transpose(1, 2), vc.cuda().transpose(1, 2),
+                                      cu_from(lens).cuda(), 0.05)
+    assert_close(got, want, TOL)
+
+
+# shapes of flash_attn_triton/flash_attn_decoding_sparse.py:409-503 and windows
+# from its sweep (:506-630)
+@pytest.mark.parametrize("gw,lw", [(256, 4096), (64, 1024), (128, 128), (64, 0), (64, 100)])
+def test_window_sparse_decode(gw, lw):
+    import tritonops_amd as ta
+
+    Hq, Hkv, D, dtype = 24, 4, 128, torch.float16
+    lens = torch.tensor([512, 2561, 8192, 0, 1, 3, 64, 200], dtype=torch.int32)
+    B, L = len(lens), int(lens.max())
+    q = randn((B, Hq, D), 1, dtype)
+    k, v = _kv(B, L, Hkv, D, dtype, 2)
+    want = orc.flash_attn_sparse_decoding_torch(q, k, v, lens, gw, lw, faithful=False)
+    got = ta.flash_attention_sparse_decoding(q.cuda(), k.cuda(), v.cuda(), cu_from(lens).cuda(), gw, lw)
+    assert_close(got, want, TOL)
+    faithful = orc.flash_attn_sparse_decoding_torch(q, k, v, lens, gw, lw, faithful=True)
+    assert_close(got, faithful, TOL)
+
+
+def test_window_sparse_decode_rejects_bad_global_window():
+    import tritonops_amd as ta
+
+    q = randn((1, 2, 64), 1).cuda()
+    k = randn((1, 64, 2, 64), 2).cuda()
+    with pytest.raises(AssertionError):
+        ta.flash_attention_sparse_decoding(q, k, k, torch.tensor([0, 64], dtype=torch.int32).cuda(), 512, 512)
+
+
+@pytest.mark.parametrize("top_k", [1, 7, 32])
+def test_block_index_decode(top_k):
+    import tritonops_amd as ta
+
+    B, Hq, Hkv, D = 3, 8, 2, 128
+    lens = torch.tensor([4096, 4000, 2049], dtype=torch.int32)
+    L = 4096
+    q = randn((B, Hq, D), 1)
+    k, v = _kv(B, L, Hkv, D, torch.bfloat16, 2)
+    g = torch.Generator().manual_seed(5)
+    idx = torch.empty(B, Hkv, top_k, dtype=torch.int32)
+    for b in range(B):
+        nblk = (int(lens[b]) + 63) // 64
+        for h in range(Hkv):
+            idx[b, h] = torch.sort(torch.randperm(nblk, generator=g)[:top_k]).values
+    want = orc.block_sparse_decoding(q, k, v, lens, idx, faithful=False)
+    got = ta.flash_attention_sparse_decoding(q.cuda(), k.cuda(), v.cuda(), None, seq_lens=lens.cuda(),
+                                             block_indices=idx.cuda())
+    assert_close(got, want, TOL)
+    # all blocks listed == dense decoding
+    if top_k == 32:
+        full = torch.arange(64, dtype=torch.int32).expand(B, Hkv, 64).contiguous()
+        cnt = ((lens + 63) // 64)[:, None].expand(B, Hkv).contiguous()
+        dense = ta.flash_attention_decoding(q.cuda(), k.cuda(), v.cuda(), None, seq_lens=lens.cuda())
+        got_all = ta.flash_attention_sparse_decoding(q.cuda(), k.cuda(), v.cuda(), None, seq_lens=lens.cuda(),
+                                                     block_indices=full.cuda(), block_counts=cnt.cuda(),
+                                                     include_last_block=False)
+        assert_close(got_all, dense, 4e-3)
+
+
+def test_full_size_decode_properties():
+    """Benchmark shape B64 Hq32 Hkv8 L<=32768 D128: a few sequences against the
+    oracle, and constant-V invariance (softmax weights sum to one)."""
+    import tritonops_amd as ta
+
+    B, Hq, Hkv, L, D = 64, 32, 8, 32768, 128
+    g = torch.Generator(device="cuda").manual_seed(0)
+    kc = torch.randn((B, Hkv, L, D), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    vc = torch.randn((B, Hkv, L, D), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    q = torch.randn((B, Hq, D), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    lens = torch.randint(16384, 32769, (B,), generator=torch.Generator().manual_seed(1), dtype=torch.int32)
+    got = ta.flash_attention_decoding(q, kc.transpose(1, 2), vc.transpose(1, 2), None, seq_lens=lens.cuda())
+    for b in (0, 31, 63):
+        want = orc.flash_attn_decoding_torch(q[b:b + 1].cpu(), kc[b:b + 1].transpose(1, 2).cpu(),
+                                             vc[b:b + 1].transpose(1, 2).cpu(), lens[b:b + 1], faithful=False)
+        assert_close(got[b:b + 1], want, TOL)
+    vc.fill_(0.5)
+    got = ta.flash_attention_decoding(q, kc.transpose(1, 2), vc.transpose(1, 2), None, seq_lens=lens.cuda())
+    assert (got.float() - 0.5).abs().max().item() <= 4e-3

@@ -1,0 +1,12 @@
+"""MI355X-native attention forward path with the call signatures of
+rookie-joe/TritonOps' flash_attn_triton package."""
+from .ops import (  # noqa: F401
+    LOG2E,
+    flash_attention,
+    flash_attention_decoding,
+    flash_attention_sparse_decoding,
+    flash_attn_sparse_triton,
+    flash_attn_triton,
+    flash_attn_triton_fwd,
+)
+from . import masks  # noqa: F401

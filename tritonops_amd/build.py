@@ -1,0 +1,62 @@
+"""Build libmi_attn.so (HIP kernels + C ABI) for gfx950 with plain hipcc.
+
+Usage: python -m tritonops_amd.build [--jobs N] [--keep-temps]
+The library is written next to this file so that it travels with the package.
+"""
+import argparse
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ_DIR = os.path.join(CSRC, "build")
+LIB_PATH = os.path.join(HERE, "libmi_attn.so")
+SOURCES = ["api.cpp", "prefill.hip", "decode.hip"]
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-Wall",
+    "-Wno-unused-function",
+    # packed-FP32 VALU forms are kept out of every kernel of this library
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _compile(src, extra):
+    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+    cmd = [HIPCC, "-x", "hip", *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in r.stderr.splitlines() if noise not in l)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s" % (src, err))
+    if err.strip():
+        sys.stderr.write(err + "\n")
+    return obj
+
+
+def build(jobs=4, keep_temps=False, verbose=True):
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    extra = ["-save-temps=obj"] if keep_temps else []
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(lambda s: _compile(s, extra), SOURCES))
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stderr)
+    if verbose:
+        print("built", LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--jobs", type=int, default=4)
+    ap.add_argument("--keep-temps", action="store_true")
+    a = ap.parse_args()
+    build(a.jobs, a.keep_temps)

@@ -1,0 +1,327 @@
+// C ABI of the library: host-side validation, launch geometry, error text.
+// Nothing in this file touches the device except the final kernel launches.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/mi_attn.h"
+#include "kernels.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+bool mult8(int64_t s) { return (s % 8) == 0; }
+
+int check_common(int dtype, int head_dim, int batch, int hq, int hkv, int max_seqlen, float scale) {
+  if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_F16) return fail(MI_ERR_DTYPE, "dtype %d is not bf16(0)/f16(1)", dtype);
+  if (head_dim != 64 && head_dim != 96 && head_dim != 128)
+    return fail(MI_ERR_HEAD_DIM, "head_dim %d not in {64, 96, 128}", head_dim);
+  if (hq <= 0 || hkv <= 0 || hq % hkv != 0)
+    return fail(MI_ERR_GQA, "heads_q %d must be a positive multiple of heads_kv %d", hq, hkv);
+  if (batch <= 0) return fail(MI_ERR_SHAPE, "batch %d must be positive", batch);
+  if (max_seqlen < 0) return fail(MI_ERR_SHAPE, "max_seqlen %d is negative", max_seqlen);
+  if (!std::isfinite(scale) || scale <= 0.f) return fail(MI_ERR_SCALE, "scale_log2 %g must be finite and > 0", (double)scale);
+  return MI_OK;
+}
+
+template <typename A>
+int check_qkvo(const A* a) {
+  if (!a->q || !a->k || !a->v || !a->o) return fail(MI_ERR_NULL_POINTER, "q, k, v and o must be non-NULL");
+  if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->o))
+    return fail(MI_ERR_ALIGNMENT, "q, k, v and o must be 16-byte aligned");
+  return MI_OK;
+}
+
+template <typename A>
+int check_prefill_strides(const A* a) {
+  const int64_t s[] = {a->q_stride_s, a->q_stride_h, a->k_stride_s, a->k_stride_h,
+                       a->v_stride_s, a->v_stride_h, a->o_stride_s, a->o_stride_h};
+  for (int64_t x : s)
+    if (!mult8(x)) return fail(MI_ERR_STRIDE, "q/k/v/o strides must be multiples of 8 elements (got %lld)", (long long)x);
+  if (!a->cu_seqlens) {
+    const int64_t sb[] = {a->q_stride_b, a->k_stride_b, a->v_stride_b, a->o_stride_b};
+    for (int64_t x : sb)
+      if (!mult8(x)) return fail(MI_ERR_STRIDE, "batch strides must be multiples of 8 elements (got %lld)", (long long)x);
+  }
+  return MI_OK;
+}
+
+template <typename A>
+void fill_prefill(const A* a, mi::PrefillParams& p, int rows_per_wg) {
+  std::memset(&p, 0, sizeof(p));
+  p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o; p.lse = a->lse;
+  p.q_sb = a->q_stride_b; p.q_ss = a->q_stride_s; p.q_sh = a->q_stride_h;
+  p.k_sb = a->k_stride_b; p.k_ss = a->k_stride_s; p.k_sh = a->k_stride_h;
+  p.v_sb = a->v_stride_b; p.v_ss = a->v_stride_s; p.v_sh = a->v_stride_h;
+  p.o_sb = a->o_stride_b; p.o_ss = a->o_stride_s; p.o_sh = a->o_stride_h;
+  p.lse_sb = a->lse_stride_b; p.lse_ss = a->lse_stride_s; p.lse_sh = a->lse_stride_h;
+  p.cu = a->cu_seqlens;
+  p.batch = a->batch; p.hq = a->heads_q; p.hkv = a->heads_kv; p.max_seqlen = a->max_seqlen;
+  p.n_qtiles = (a->max_seqlen + rows_per_wg - 1) / rows_per_wg;
+  p.scale = a->scale_log2;
+  p.win_local = -1; p.win_global = -1;
+}
+
+int decode_splits(const mi_decode_args* a) {
+  if (a->block_idx) return (a->max_blocks + a->split_blocks - 1) / a->split_blocks;
+  return (a->max_seqlen + a->split_tokens - 1) / a->split_tokens;
+}
+
+void fill_decode(const mi_decode_args* a, mi::DecodeParams& p) {
+  std::memset(&p, 0, sizeof(p));
+  p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o; p.lse = a->lse;
+  p.q_sb = a->q_stride_b; p.q_sh = a->q_stride_h;
+  p.k_sb = a->k_stride_b; p.k_ss = a->k_stride_s; p.k_sh = a->k_stride_h;
+  p.v_sb = a->v_stride_b; p.v_ss = a->v_stride_s; p.v_sh = a->v_stride_h;
+  p.o_sb = a->o_stride_b; p.o_sh = a->o_stride_h;
+  p.seq_lens = a->seq_lens; p.cu = a->cu_seqlens;
+  p.batch = a->batch; p.hq = a->heads_q; p.hkv = a->heads_kv; p.max_seqlen = a->max_seqlen;
+  p.scale = a->scale_log2;
+  p.split_tokens = a->split_tokens;
+  p.n_splits = decode_splits(a);
+  p.part_o = static_cast<float*>(a->workspace);
+  p.part_lse = p.part_o + (size_t)a->batch * a->heads_q * p.n_splits * a->head_dim;
+  p.block_idx = a->block_idx; p.block_cnt = a->block_cnt;
+  p.bi_sb = a->block_idx_stride_b; p.bi_sh = a->block_idx_stride_h;
+  p.max_blocks = a->max_blocks; p.split_blocks = a->split_blocks;
+  p.win_local = a->block_idx ? a->window_local : -1;
+  p.win_global = a->block_idx ? a->window_global : -1;
+  if (!a->block_idx) { p.max_blocks = 0; p.split_blocks = 1; }
+}
+
+int launch_status(int hip_err, const char* what) {
+  if (hip_err == 0) return MI_OK;
+  return fail(MI_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(static_cast<hipError_t>(hip_err)));
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi_abi_version(void) { return MI_ATTN_ABI_VERSION; }
+const char* mi_last_error(void) { return g_err; }
+
+const char* mi_status_name(int status) {
+  switch (status) {
+    case MI_OK: return "MI_OK";
+    case MI_ERR_NULL_POINTER: return "MI_ERR_NULL_POINTER";
+    case MI_ERR_STRUCT_SIZE: return "MI_ERR_STRUCT_SIZE";
+    case MI_ERR_DTYPE: return "MI_ERR_DTYPE";
+    case MI_ERR_HEAD_DIM: return "MI_ERR_HEAD_DIM";
+    case MI_ERR_GQA: return "MI_ERR_GQA";
+    case MI_ERR_SHAPE: return "MI_ERR_SHAPE";
+    case MI_ERR_STRIDE: return "MI_ERR_STRIDE";
+    case MI_ERR_ALIGNMENT: return "MI_ERR_ALIGNMENT";
+    case MI_ERR_SCALE: return "MI_ERR_SCALE";
+    case MI_ERR_WORKSPACE: return "MI_ERR_WORKSPACE";
+    case MI_ERR_SPARSE_LAYOUT: return "MI_ERR_SPARSE_LAYOUT";
+    case MI_ERR_LAUNCH: return "MI_ERR_LAUNCH";
+    case MI_ERR_NO_DEVICE: return "MI_ERR_NO_DEVICE";
+  }
+  return "MI_ERR_UNKNOWN";
+}
+
+int mi_attn_fwd_validate(const mi_attn_fwd_args* a) {
+  if (!a) return fail(MI_ERR_NULL_POINTER, "args is NULL");
+  if (a->struct_size != sizeof(mi_attn_fwd_args))
+    return fail(MI_ERR_STRUCT_SIZE, "mi_attn_fwd_args.struct_size %u != %zu", a->struct_size, sizeof(mi_attn_fwd_args));
+  int rc = check_common(a->dtype, a->head_dim, a->batch, a->heads_q, a->heads_kv, a->max_seqlen, a->scale_log2);
+  if (rc) return rc;
+  if ((rc = check_qkvo(a))) return rc;
+  if ((rc = check_prefill_strides(a))) return rc;
+  if (a->causal != 0 && a->causal != 1) return fail(MI_ERR_SHAPE, "causal must be 0 or 1");
+  const long long wgs = (long long)((a->max_seqlen + mi::kDenseRows - 1) / mi::kDenseRows) * a->heads_q * a->batch;
+  if (wgs > 0x7fffffffLL) return fail(MI_ERR_SHAPE, "grid of %lld workgroups is too large", wgs);
+  return MI_OK;
+}
+
+int mi_attn_fwd(const mi_attn_fwd_args* a, void* stream) {
+  int rc = mi_attn_fwd_validate(a);
+  if (rc) return rc;
+  if (a->max_seqlen == 0) return MI_OK;
+  mi::PrefillParams p;
+  fill_prefill(a, p, mi::kDenseRows);
+  p.causal = a->causal;
+  return launch_status(mi::launch_prefill_dense(p, a->dtype, a->head_dim, static_cast<hipStream_t>(stream)), "mi_attn_fwd");
+}
+
+int mi_attn_fwd_blocksparse_validate(const mi_attn_sparse_args* a) {
+  if (!a) return fail(MI_ERR_NULL_POINTER, "args is NULL");
+  if (a->struct_size != sizeof(mi_attn_sparse_args))
+    return fail(MI_ERR_STRUCT_SIZE, "mi_attn_sparse_args.struct_size %u != %zu", a->struct_size, sizeof(mi_attn_sparse_args));
+  int rc = check_common(a->dtype, a->head_dim, a->batch, a->heads_q, a->heads_kv, a->max_seqlen, a->scale_log2);
+  if (rc) return rc;
+  if ((rc = check_qkvo(a))) return rc;
+  if ((rc = check_prefill_strides(a))) return rc;
+  if (!a->row_ptr || !a->col_idx) return fail(MI_ERR_NULL_POINTER, "row_ptr and col_idx must be non-NULL");
+  if (a->block_size != MI_ATTN_BLOCK) return fail(MI_ERR_SPARSE_LAYOUT, "block_size %d must be %d", a->block_size, MI_ATTN_BLOCK);
+  if (a->row_ptr_stride_b < 0 || a->row_ptr_stride_h < 0 || a->col_idx_stride_b < 0 || a->col_idx_stride_h < 0)
+    return fail(MI_ERR_SPARSE_LAYOUT, "mask strides must be >= 0");
+  if ((a->window_local < 0) != (a->window_global < 0) || a->window_local < -1 || a->window_global < -1)
+    return fail(MI_ERR_SPARSE_LAYOUT, "window_local/window_global must both be -1 or both be >= 0");
+  const long long wgs = (long long)((a->max_seqlen + mi::kSparseRows - 1) / mi::kSparseRows) * a->heads_q * a->batch;
+  if (wgs > 0x7fffffffLL) return fail(MI_ERR_SHAPE, "grid of %lld workgroups is too large", wgs);
+  return MI_OK;
+}
+
+int mi_attn_fwd_blocksparse(const mi_attn_sparse_args* a, void* stream) {
+  int rc = mi_attn_fwd_blocksparse_validate(a);
+  if (rc) return rc;
+  if (a->max_seqlen == 0) return MI_OK;
+  mi::PrefillParams p;
+  fill_prefill(a, p, mi::kSparseRows);
+  p.causal = 1;
+  p.row_ptr = a->row_ptr; p.col_idx = a->col_idx;
+  p.rp_sb = a->row_ptr_stride_b; p.rp_sh = a->row_ptr_stride_h;
+  p.ci_sb = a->col_idx_stride_b; p.ci_sh = a->col_idx_stride_h;
+  p.win_local = a->window_local; p.win_global = a->window_global;
+  return launch_status(mi::launch_prefill_sparse(p, a->dtype, a->head_dim, static_cast<hipStream_t>(stream)), "mi_attn_fwd_blocksparse");
+}
+
+static int decode_validate_shape(const mi_decode_args* a) {
+  if (!a) return fail(MI_ERR_NULL_POINTER, "args is NULL");
+  if (a->struct_size != sizeof(mi_decode_args))
+    return fail(MI_ERR_STRUCT_SIZE, "mi_decode_args.struct_size %u != %zu", a->struct_size, sizeof(mi_decode_args));
+  int rc = check_common(a->dtype, a->head_dim, a->batch, a->heads_q, a->heads_kv, a->max_seqlen, a->scale_log2);
+  if (rc) return rc;
+  if (a->heads_q / a->heads_kv > 32)
+    return fail(MI_ERR_GQA, "at most 32 query heads per kv head (got %d)", a->heads_q / a->heads_kv);
+  if (a->block_idx) {
+    if (a->block_size != MI_ATTN_BLOCK) return fail(MI_ERR_SPARSE_LAYOUT, "block_size %d must be %d", a->block_size, MI_ATTN_BLOCK);
+    if (a->max_blocks <= 0 || a->split_blocks <= 0)
+      return fail(MI_ERR_SPARSE_LAYOUT, "max_blocks %d and split_blocks %d must be positive", a->max_blocks, a->split_blocks);
+    if (a->block_idx_stride_b < 0 || a->block_idx_stride_h < 0)
+      return fail(MI_ERR_SPARSE_LAYOUT, "block_idx strides must be >= 0");
+    if ((a->window_local < 0) != (a->window_global < 0) || a->window_local < -1 || a->window_global < -1)
+      return fail(MI_ERR_SPARSE_LAYOUT, "window_local/window_global must both be -1 or both be >= 0");
+  } else {
+    if (a->split_tokens <= 0 || a->split_tokens % 64 != 0)
+      return fail(MI_ERR_WORKSPACE, "split_tokens %d must be a positive multiple of 64", a->split_tokens);
+  }
+  if (decode_splits(a) > 65535) return fail(MI_ERR_WORKSPACE, "more than 65535 splits per sequence");
+  if (a->heads_kv > 65535 || a->batch > 65535 || a->heads_q > 0x7fffffff / 2)
+    return fail(MI_ERR_SHAPE, "batch / head count exceeds the launch grid limits");
+  return MI_OK;
+}
+
+int mi_decode_num_splits(const mi_decode_args* a) {
+  int rc = decode_validate_shape(a);
+  if (rc) return rc;
+  return decode_splits(a);
+}
+
+size_t mi_decode_workspace_bytes(const mi_decode_args* a) {
+  if (decode_validate_shape(a)) return 0;
+  return (size_t)a->batch * a->heads_q * decode_splits(a) * (a->head_dim + 1) * sizeof(float);
+}
+
+int mi_decode_choose_split_tokens(int batch, int heads_kv, int max_seqlen, int num_cus) {
+  // One wavefront per (chunk, kv-head, sequence); aim for ~16 wavefronts per
+  // compute unit's worth of chunks so the tail is short, with chunks no shorter
+  // than 256 tokens (partials stay < 2 % of the KV bytes) and no longer than 4096.
+  if (batch <= 0 || heads_kv <= 0 || max_seqlen <= 0) return 64;
+  if (num_cus <= 0) num_cus = 256;
+  const long long units = (long long)batch * heads_kv;
+  const long long want = 16LL * num_cus;
+  long long splits = (want + units - 1) / units;
+  if (splits < 1) splits = 1;
+  long long tokens = (max_seqlen + splits - 1) / splits;
+  tokens = (tokens + 63) / 64 * 64;
+  if (tokens < 256) tokens = 256;
+  if (tokens > 4096) tokens = 4096;
+  return (int)tokens;
+}
+
+int mi_decode_validate(const mi_decode_args* a) {
+  int rc = decode_validate_shape(a);
+  if (rc) return rc;
+  if (!a->q || !a->k || !a->v || !a->o) return fail(MI_ERR_NULL_POINTER, "q, k, v and o must be non-NULL");
+  if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v))
+    return fail(MI_ERR_ALIGNMENT, "q, k and v must be 16-byte aligned");
+  if ((a->seq_lens == nullptr) == (a->cu_seqlens == nullptr))
+    return fail(MI_ERR_NULL_POINTER, "exactly one of seq_lens / cu_seqlens must be non-NULL");
+  const int64_t s[] = {a->q_stride_b, a->q_stride_h, a->k_stride_b, a->k_stride_s, a->k_stride_h,
+                       a->v_stride_b, a->v_stride_s, a->v_stride_h};
+  for (int64_t x : s)
+    if (!mult8(x)) return fail(MI_ERR_STRIDE, "q/k/v strides must be multiples of 8 elements (got %lld)", (long long)x);
+  if (!a->workspace) return fail(MI_ERR_NULL_POINTER, "workspace is NULL");
+  if (!aligned16(a->workspace)) return fail(MI_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
+  const size_t need = mi_decode_workspace_bytes(a);
+  if (a->workspace_bytes < need)
+    return fail(MI_ERR_WORKSPACE, "workspace_bytes %zu < required %zu", a->workspace_bytes, need);
+  return MI_OK;
+}
+
+int mi_decode_splitkv(const mi_decode_args* a, void* stream) {
+  int rc = mi_decode_validate(a);
+  if (rc) return rc;
+  if (a->max_seqlen == 0) return MI_OK;
+  mi::DecodeParams p;
+  fill_decode(a, p);
+  return launch_status(mi::launch_decode_splitkv(p, a->dtype, a->head_dim, static_cast<hipStream_t>(stream)), "mi_decode_splitkv");
+}
+
+int mi_decode_merge(const mi_decode_args* a, void* stream) {
+  int rc = mi_decode_validate(a);
+  if (rc) return rc;
+  mi::DecodeParams p;
+  fill_decode(a, p);
+  if (a->max_seqlen == 0) p.n_splits = 0;
+  return launch_status(mi::launch_decode_merge(p, a->dtype, a->head_dim, static_cast<hipStream_t>(stream)), "mi_decode_merge");
+}
+
+int mi_decode(const mi_decode_args* a, void* stream) {
+  int rc = mi_decode_splitkv(a, stream);
+  if (rc) return rc;
+  return mi_decode_merge(a, stream);
+}
+
+int mi_time_launches(int kind, const void* args, void* stream, int warmup, int iters, float* ms_per_launch) {
+  if (!args || !ms_per_launch) return fail(MI_ERR_NULL_POINTER, "args / ms_per_launch is NULL");
+  if (iters <= 0 || warmup < 0 || kind < 0 || kind > 4) return fail(MI_ERR_SHAPE, "bad kind / warmup / iters");
+  auto once = [&]() -> int {
+    switch (kind) {
+      case 0: return mi_attn_fwd(static_cast<const mi_attn_fwd_args*>(args), stream);
+      case 1: return mi_attn_fwd_blocksparse(static_cast<const mi_attn_sparse_args*>(args), stream);
+      case 2: return mi_decode(static_cast<const mi_decode_args*>(args), stream);
+      case 3: return mi_decode_splitkv(static_cast<const mi_decode_args*>(args), stream);
+      default: return mi_decode_merge(static_cast<const mi_decode_args*>(args), stream);
+    }
+  };
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  for (int i = 0; i < warmup; ++i) {
+    int rc = once();
+    if (rc) return rc;
+  }
+  hipEvent_t e0, e1;
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)
+    return fail(MI_ERR_NO_DEVICE, "hipEventCreate failed");
+  int rc = MI_OK;
+  (void)hipEventRecord(e0, s);
+  for (int i = 0; i < iters && rc == MI_OK; ++i) rc = once();
+  (void)hipEventRecord(e1, s);
+  hipError_t e = hipEventSynchronize(e1);
+  float ms = 0.f;
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (rc) return rc;
+  if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "timing failed: %s", hipGetErrorString(e));
+  *ms_per_launch = ms / iters;
+  return MI_OK;
+}
+
+}  // extern "C"

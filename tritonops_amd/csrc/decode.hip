@@ -1,0 +1,218 @@
+// Single-query (decoding) attention for gfx950: split-KV pass + LSE merge pass,
+// dense and block-sparse.
+//
+// Replaces flash_attn_decoding_kernel / flash_attn_decoding_correction_kernel
+// of flash_attn_triton/flash_attn_decoding.py:9-122,:126-210 and their sparse
+// twins in flash_attn_triton/flash_attn_decoding_sparse.py:10-127,:131-219.
+//
+// Pass 1: one wavefront (= one workgroup) per (chunk, kv-head, sequence).  The
+// G = hq/hkv query heads that share the kv-head sit in the first G of the 32
+// query columns of the same S^T = K.Q^T / O^T = V^T.P^T MFMA pipeline the
+// prefill kernel uses, so each K/V byte is fetched once for the whole group
+// (the reference launches one program per q-head and re-reads KV G times,
+// flash_attn_decoding.py:42-45,264-268) and the dot products cost no VALU
+// work.  KV streams global -> registers -> wave-private LDS in 32-key tiles
+// with fully coalesced 16-byte loads; no barriers are needed because a single
+// wave's LDS operations execute in order.  Partials are fp32 (the reference
+// rounds them to the input dtype, :249-251).
+// Pass 2: per (sequence, q-head) merge  o = sum_c o_c 2^(lse_c - lse).
+#include "kernels.h"
+#include "tile_core.h"
+
+namespace mi {
+namespace {
+
+constexpr int kDecTile = 32;
+
+template <typename T, int D>
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2)))
+decode_splitkv_kernel(const DecodeParams p) {
+  using G = RowGeom<D>;
+  constexpr int TILEB = kDecTile * G::ROWB;
+  constexpr int NCHUNK = kDecTile * G::NCH;
+  constexpr int LOADS = (NCHUNK + 63) / 64;
+
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * TILEB];
+  unsigned char* sK = smem;
+  unsigned char* sV = smem + TILEB;
+
+  const int lane = threadIdx.x;
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int len = p.seq_lens ? p.seq_lens[b] : p.cu[b + 1] - p.cu[b];
+  const int gqa = p.hq / p.hkv;
+  const bool sparse = p.block_idx != nullptr;
+
+  int n_tiles, t_begin = 0;
+  const int32_t* blist = nullptr;
+  if (sparse) {
+    const int cnt = p.block_cnt ? min(p.block_cnt[b * p.hkv + kvh], p.max_blocks) : p.max_blocks;
+    const int b0 = split * p.split_blocks;
+    if (b0 >= cnt || len <= 0) return;
+    blist = p.block_idx + b * p.bi_sb + kvh * p.bi_sh + b0;
+    n_tiles = 2 * min(cnt - b0, p.split_blocks);
+  } else {
+    t_begin = split * p.split_tokens;
+    if (t_begin >= len) return;
+    n_tiles = (min(len, t_begin + p.split_tokens) - t_begin + kDecTile - 1) / kDecTile;
+  }
+  auto tile_base = [&](int i) -> int {
+    return sparse ? blist[i >> 1] * 64 + (i & 1) * kDecTile : t_begin + i * kDecTile;
+  };
+
+  const T* kp = reinterpret_cast<const T*>(p.k) + b * p.k_sb + kvh * p.k_sh;
+  const T* vp = reinterpret_cast<const T*>(p.v) + b * p.v_sb + kvh * p.v_sh;
+
+  LaneCtx<D> lc;
+  lc.init(lane);
+
+  // Q^T operand: column lq is q-head kvh*gqa + lq, columns >= gqa are zero.
+  i32x4 Qf[G::KSTEPS];
+  {
+    const T* qr = reinterpret_cast<const T*>(p.q) + b * p.q_sb +
+                  (int64_t)(kvh * gqa + min(lc.lq, gqa - 1)) * p.q_sh + 8 * lc.lh;
+#pragma unroll
+    for (int c = 0; c < G::KSTEPS; ++c) {
+      i32x4 t = *reinterpret_cast<const i32x4*>(qr + 16 * c);
+      Qf[c] = lc.lq < gqa ? t : (i32x4){0, 0, 0, 0};
+    }
+  }
+
+  f32x16 O[G::NDB];
+#pragma unroll
+  for (int db = 0; db < G::NDB; ++db) O[db] = (f32x16){0};
+  float m = -INFINITY, l = 0.f;
+
+  i32x4 kreg[LOADS], vreg[LOADS];
+  auto gload = [&](int base) {
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const int idx = lane + i * 64;
+      if (NCHUNK % 64 == 0 || idx < NCHUNK) {
+        const int row = idx / G::NCH, ch = idx % G::NCH;
+        const int64_t kr = max(0, min(base + row, len - 1));
+        kreg[i] = *reinterpret_cast<const i32x4*>(kp + kr * p.k_ss + ch * 8);
+        vreg[i] = *reinterpret_cast<const i32x4*>(vp + kr * p.v_ss + ch * 8);
+      }
+    }
+  };
+  auto lstore = [&]() {
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const int idx = lane + i * 64;
+      if (NCHUNK % 64 == 0 || idx < NCHUNK) {
+        const int row = idx / G::NCH, ch = idx % G::NCH;
+        lds_store_k<D>(sK, row, ch, kreg[i]);
+        lds_store_v<D>(sV, row, ch, vreg[i]);
+      }
+    }
+  };
+
+  const int wl = p.win_local, wg = p.win_global;
+  gload(tile_base(0));
+  lstore();
+  for (int it = 0; it < n_tiles; ++it) {
+    const int base = tile_base(it);
+    const bool more = it + 1 < n_tiles;
+    if (more) gload(tile_base(it + 1));
+    bool need_mask = base + kDecTile > len;
+    if (wl >= 0) need_mask = need_mask || !((base + kDecTile - 1 < wg) || (base >= len - wl));
+    auto allowed = [&](int key_in_tile) -> bool {
+      const int key = base + key_in_tile;
+      bool ok = key < len;
+      if (wl >= 0) ok = ok && (key < wg || key >= len - wl);
+      return ok;
+    };
+    compute_tile<T, D, 1>(sK, sV, lc, Qf, O, m, l, p.scale, need_mask, allowed);
+    if (more) lstore();
+  }
+
+  const float l_tot = sum_with_other_half(l);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  if (lc.lq < gqa) {
+    const int h = kvh * gqa + lc.lq;
+    const int64_t slot = ((int64_t)b * p.hq + h) * p.n_splits + split;
+    if (lc.lh == 0) p.part_lse[slot] = l_tot > 0.f ? m + fast_log2(l_tot) : -INFINITY;
+    float* po = p.part_o + slot * D;
+#pragma unroll
+    for (int db = 0; db < G::NDB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float4 w = {O[db][4 * g] * inv, O[db][4 * g + 1] * inv, O[db][4 * g + 2] * inv,
+                    O[db][4 * g + 3] * inv};
+        *reinterpret_cast<float4*>(po + 32 * db + 8 * g + 4 * lc.lh) = w;
+      }
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(128)
+decode_merge_kernel(const DecodeParams p, int D) {
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int d = threadIdx.x;
+  const int len = p.seq_lens ? p.seq_lens[b] : p.cu[b + 1] - p.cu[b];
+  int nvalid;
+  if (p.block_idx) {
+    const int kvh = h / (p.hq / p.hkv);
+    const int cnt = p.block_cnt ? min(p.block_cnt[b * p.hkv + kvh], p.max_blocks) : p.max_blocks;
+    nvalid = len > 0 ? (cnt + p.split_blocks - 1) / p.split_blocks : 0;
+  } else {
+    nvalid = (len + p.split_tokens - 1) / p.split_tokens;
+  }
+  nvalid = max(0, min(nvalid, p.n_splits));
+  const int64_t slot0 = ((int64_t)b * p.hq + h) * p.n_splits;
+  const float* pl = p.part_lse + slot0;
+
+  float M = -INFINITY;
+  for (int c = 0; c < nvalid; ++c) M = fmaxf(M, pl[c]);
+  float den = 0.f, acc = 0.f;
+  if (M > -INFINITY && d < D) {
+    const float* po = p.part_o + slot0 * D + d;
+    for (int c = 0; c < nvalid; ++c) {
+      const float w = fast_exp2(pl[c] - M);
+      den += w;
+      acc += w * po[(int64_t)c * D];
+    }
+  }
+  if (d < D) {
+    T* op = reinterpret_cast<T*>(p.o) + b * p.o_sb + h * p.o_sh;
+    op[d] = (T)(den > 0.f ? acc / den : 0.f);
+  }
+  if (d == 0 && p.lse) p.lse[(int64_t)b * p.hq + h] = den > 0.f ? M + fast_log2(den) : -INFINITY;
+}
+
+template <typename T, int D>
+int launch_split(const DecodeParams& p, hipStream_t s) {
+  dim3 grid(p.n_splits, p.hkv, p.batch);
+  hipLaunchKernelGGL((decode_splitkv_kernel<T, D>), grid, dim3(64), 0, s, p);
+  return (int)hipGetLastError();
+}
+
+}  // namespace
+
+int launch_decode_splitkv(const DecodeParams& p, int dtype, int head_dim, hipStream_t s) {
+  if (dtype == 0) {
+    switch (head_dim) {
+      case 64: return launch_split<__bf16, 64>(p, s);
+      case 96: return launch_split<__bf16, 96>(p, s);
+      case 128: return launch_split<__bf16, 128>(p, s);
+    }
+  } else {
+    switch (head_dim) {
+      case 64: return launch_split<_Float16, 64>(p, s);
+      case 96: return launch_split<_Float16, 96>(p, s);
+      case 128: return launch_split<_Float16, 128>(p, s);
+    }
+  }
+  return (int)hipErrorInvalidValue;
+}
+
+int launch_decode_merge(const DecodeParams& p, int dtype, int head_dim, hipStream_t s) {
+  dim3 grid(p.hq, p.batch);
+  if (dtype == 0)
+    hipLaunchKernelGGL((decode_merge_kernel<__bf16>), grid, dim3(128), 0, s, p, head_dim);
+  else
+    hipLaunchKernelGGL((decode_merge_kernel<_Float16>), grid, dim3(128), 0, s, p, head_dim);
+  return (int)hipGetLastError();
+}
+
+}  // namespace mi

@@ -1,0 +1,64 @@
+// Host-visible launch interface between the C ABI layer (api.cpp) and the HIP
+// translation units.  Everything here is already validated by the caller.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mi {
+
+struct PrefillParams {
+  const void *q, *k, *v;
+  void* o;
+  float* lse;  // may be null
+  int64_t q_sb, q_ss, q_sh;
+  int64_t k_sb, k_ss, k_sh;
+  int64_t v_sb, v_ss, v_sh;
+  int64_t o_sb, o_ss, o_sh;
+  int64_t lse_sb, lse_ss, lse_sh;
+  const int32_t* cu;  // null => batched
+  // block-sparse only
+  const int32_t* row_ptr;
+  const int32_t* col_idx;
+  int64_t rp_sb, rp_sh, ci_sb, ci_sh;
+  int32_t batch, hq, hkv, max_seqlen;
+  int32_t n_qtiles;  // ceil(max_seqlen / rows per workgroup)
+  int32_t causal;
+  int32_t win_local, win_global;  // -1 => off
+  float scale;                    // log2 domain
+};
+
+struct DecodeParams {
+  const void *q, *k, *v;
+  void* o;
+  float* lse;  // may be null
+  int64_t q_sb, q_sh;
+  int64_t k_sb, k_ss, k_sh;
+  int64_t v_sb, v_ss, v_sh;
+  int64_t o_sb, o_sh;
+  const int32_t* seq_lens;  // one of the two
+  const int32_t* cu;
+  int32_t batch, hq, hkv, max_seqlen;
+  float scale;
+  int32_t split_tokens;  // dense chunk, multiple of 64
+  int32_t n_splits;      // chunks per sequence (grid.x)
+  float* part_o;         // [batch][hq][n_splits][D]
+  float* part_lse;       // [batch][hq][n_splits]
+  // block-sparse
+  const int32_t* block_idx;  // null => dense
+  const int32_t* block_cnt;
+  int64_t bi_sb, bi_sh;
+  int32_t max_blocks, split_blocks;
+  int32_t win_local, win_global;
+};
+
+// dtype: 0 bf16, 1 f16.  head_dim in {64, 96, 128}.  Return hipError_t as int.
+int launch_prefill_dense(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);
+int launch_prefill_sparse(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);
+int launch_decode_splitkv(const DecodeParams& p, int dtype, int head_dim, hipStream_t s);
+int launch_decode_merge(const DecodeParams& p, int dtype, int head_dim, hipStream_t s);
+
+// Query rows per workgroup of the two prefill kernels.
+constexpr int kDenseRows = 128;
+constexpr int kSparseRows = 64;
+
+}  // namespace mi

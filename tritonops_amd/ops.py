@@ -1,0 +1,366 @@
+"""Drop-in Python entry points of the attention forward path.
+
+Names, positional arguments and semantics follow the reference launchers
+(citations per function, paths relative to the reference checkout); the work
+is done by the HIP kernels of libmi_attn.so reached through its C ABI.  There
+is no fallback: without the built library every call raises.
+"""
+import ctypes as C
+import math
+
+import torch
+
+from . import _lib
+from . import masks as _masks
+
+LOG2E = 1.4426950408889634
+_NUM_CUS = 256
+
+
+def _dtype_tag(t):
+    if t.dtype == torch.bfloat16:
+        return _lib.MI_DTYPE_BF16
+    if t.dtype == torch.float16:
+        return _lib.MI_DTYPE_F16
+    raise TypeError("attention inputs must be bfloat16 or float16, got %s" % t.dtype)
+
+
+def _require_gpu(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("tritonops_amd runs on the GPU only (tensor on %s); there is no CPU path" % t.device)
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _inner_contig(t):
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def _max_len(cu_seq_lens, max_seq_len):
+    if max_seq_len is not None:
+        return int(max_seq_len)
+    # same host round trip as the reference launcher
+    # (flash_attn_triton/flash_attn_triton.py:621)
+    return int((cu_seq_lens[1:] - cu_seq_lens[:-1]).max().item())
+
+
+def _fill_qkvo(a, q, k, v, o, lse, packed):
+    """q/k/v/o given as [X, S, H, D] views (X = 1 packed, X = B batched)."""
+    a.q, a.k, a.v, a.o, a.lse = _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse)
+    for name, t in (("q", q), ("k", k), ("v", v), ("o", o)):
+        setattr(a, name + "_stride_b", 0 if packed else t.stride(0))
+        setattr(a, name + "_stride_s", t.stride(1))
+        setattr(a, name + "_stride_h", t.stride(2))
+    if lse is not None:
+        a.lse_stride_b = 0 if packed else lse.stride(0)
+        a.lse_stride_s = lse.stride(1)
+        a.lse_stride_h = lse.stride(2)
+
+
+def _dense_fwd(q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, want_lse=True, bhsd=False):
+    """q,k,v as [X, S, H, D] (see _fill_qkvo). Returns (o, lse[X, S, H]); with
+    `bhsd` the outputs own [X, H, S, D] / [X, H, S] memory and are returned as
+    [X, S, H, ...] views of it."""
+    _require_gpu(q, k, v, cu_seq_lens)
+    lib = _lib.load()
+    q, k, v = _inner_contig(q), _inner_contig(k), _inner_contig(v)
+    packed = cu_seq_lens is not None
+    X, S, Hq, D = q.shape
+    if k.shape[-1] != D or v.shape[-1] != D:
+        raise ValueError("q, k and v must share head_dim (got %d, %d, %d)" % (D, k.shape[-1], v.shape[-1]))
+    if bhsd:
+        o = torch.empty((X, Hq, S, D), device=q.device, dtype=q.dtype).transpose(1, 2)
+        lse = torch.empty((X, Hq, S), device=q.device, dtype=torch.float32).transpose(1, 2) if want_lse else None
+    else:
+        o = torch.empty((X, S, Hq, D), device=q.device, dtype=q.dtype)
+        lse = torch.empty((X, S, Hq), device=q.device, dtype=torch.float32) if want_lse else None
+    a = _lib.AttnFwdArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _dtype_tag(q)
+    _fill_qkvo(a, q, k, v, o, lse, packed)
+    if packed:
+        if X != 1:
+            raise ValueError("packed layout expects a leading dimension of 1")
+        cu = cu_seq_lens.to(torch.int32)
+        a.cu_seqlens = _ptr(cu)
+        a.batch = cu.numel() - 1
+        a.max_seqlen = min(_max_len(cu, max_seq_len), S)
+    else:
+        a.cu_seqlens = None
+        a.batch = X
+        a.max_seqlen = S
+    a.heads_q, a.heads_kv, a.head_dim = Hq, k.shape[2], D
+    a.causal = 1 if causal else 0
+    a.scale_log2 = float(scale_log2)
+    _lib.check(lib.mi_attn_fwd(C.byref(a), _stream()))
+    return o, lse
+
+
+def flash_attn_triton_fwd(q, k, v, cu_seq_lens, sm_scale, *, max_seq_len=None):
+    """Causal var-len GQA forward on packed tensors.
+
+    Same contract as flash_attn_triton_fwd in
+    flash_attn_triton/flash_attn_triton.py:595-658: q [1,T,Hq,D], k/v
+    [1,T,Hkv,D], cu_seq_lens [B+1]; `sm_scale` already contains log2(e)
+    (:839).  Returns (o [1,T,Hq,D], lse [1,T,Hq] fp32, base 2).  Rows outside
+    every sequence are left unwritten (the reference zero-fills them).
+    `max_seq_len` skips the host sync that sizes the grid (:621).
+    """
+    return _dense_fwd(q, k, v, cu_seq_lens, sm_scale, True, max_seq_len)
+
+
+class flash_attn_triton(torch.autograd.Function):
+    """`flash_attn_triton.apply(q, k, v, cu_seq_lens) -> o`, the autograd entry
+    of flash_attn_triton/flash_attn_triton.py:816-874.  Forward only: the
+    backward kernels (:183-593) are not part of this library yet and
+    `backward` raises."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, cu_seq_lens):
+        sm_scale = (1 / q.shape[-1]) ** 0.5 * LOG2E
+        o, lse = flash_attn_triton_fwd(q, k, v, cu_seq_lens, sm_scale)
+        ctx.save_for_backward(q, k, v, o, lse, cu_seq_lens)
+        ctx.sm_scale = sm_scale
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        raise NotImplementedError("attention backward is not implemented in tritonops_amd")
+
+
+def flash_attention(q, k, v, cu_seq_lens=None, *, causal=True, softmax_scale=None,
+                    return_lse=False, max_seq_len=None):
+    """The entry point the reference README advertises (README.md:30-31).
+
+    Packed form (cu_seq_lens given): identical to flash_attn_triton.apply —
+    q [1,T,Hq,D], k/v [1,T,Hkv,D], always per-sequence causal in the reference
+    (flash_attn_triton.py:819-846); `causal=False` is an extension.
+    Batched form (cu_seq_lens None): q [B,H,S,D], k/v [B,Hkv,S,D], the layout
+    of tutorial/4.3.multi_head_attention.py:153-194 (non-causal) and
+    tutorial/4.4.causal_attention.py (causal).
+    `softmax_scale` is in the natural base; default D^-0.5.
+    Returns o, or (o, lse2) with return_lse (lse2 [1,T,Hq] / [B,H,S]).
+    """
+    D = q.shape[-1]
+    scale = (D ** -0.5 if softmax_scale is None else float(softmax_scale)) * LOG2E
+    if cu_seq_lens is not None:
+        o, lse = _dense_fwd(q, k, v, cu_seq_lens, scale, causal, max_seq_len, return_lse)
+        return (o, lse) if return_lse else o
+    if q.dim() != 4:
+        raise ValueError("batched form expects [B, H, S, D] tensors")
+    o, lse = _dense_fwd(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), None, scale, causal,
+                        None, return_lse, bhsd=True)
+    o = o.transpose(1, 2)  # contiguous [B,H,S,D]
+    if return_lse:
+        return o, lse.transpose(1, 2)
+    return o
+
+
+def flash_attn_sparse_triton(q, k, v, cu_seqlens, softmax_scale=None, local_window_size=0,
+                             global_window_size=0, *, block_mask=None, row_ptr=None, col_idx=None,
+                             csr_strides=(0, 0, 0, 0), max_seq_len=None):
+    """Sparse causal forward on packed tensors; returns (o, lse2).
+
+    Window form — the launcher of
+    flash_attn_triton/flash_attn_sparse_attn_triton.py:237-326 (the name is the
+    one its test calls, :480): attends k <= q and (q - k < local_window_size
+    or k < global_window_size), the rule of the oracle at :422-433, applied per
+    token.  `softmax_scale` is in the natural base as in that oracle (:405-406).
+    With cu_seqlens=None the tensors are batched [B,H,S,D] (extension).
+    Block form — pass `block_mask` (bool [nq,nq] / [H,nq,nq] / [B,H,nq,nq] over
+    64-token blocks, lower triangular) or a prebuilt CSR (`row_ptr`, `col_idx`,
+    `csr_strides`); diagonal blocks are masked causally per token.
+    A query with no allowed key gets o = 0 and lse = -inf.
+    """
+    _require_gpu(q, k, v, cu_seqlens)
+    lib = _lib.load()
+    q, k, v = _inner_contig(q), _inner_contig(k), _inner_contig(v)
+    packed = cu_seqlens is not None
+    if packed:
+        X, T, Hq, D = q.shape
+        if X != 1:
+            raise ValueError("packed layout expects a leading dimension of 1")
+        cu = cu_seqlens.to(torch.int32)
+        max_len = min(_max_len(cu, max_seq_len), T)
+        o = torch.empty_like(q)
+        lse = torch.empty((1, T, Hq), device=q.device, dtype=torch.float32)
+        qv, kv, vv, ov, lv = q, k, v, o, lse
+        batch = cu.numel() - 1
+    else:
+        # batched [B,H,S,D] form (extension, same layout as flash_attention)
+        X, Hq, T, D = q.shape
+        cu = None
+        max_len = T
+        o = torch.empty((X, Hq, T, D), device=q.device, dtype=q.dtype)
+        lse = torch.empty((X, Hq, T), device=q.device, dtype=torch.float32)
+        qv, kv, vv, ov, lv = (t.transpose(1, 2) for t in (q, k, v, o, lse))
+        batch = X
+    scale = (D ** -0.5 if softmax_scale is None else float(softmax_scale)) * LOG2E
+    nqb = max((max_len + _masks.BLOCK - 1) // _masks.BLOCK, 1)
+    wl = wg = -1
+    if row_ptr is None:
+        if block_mask is None:
+            wl, wg = int(local_window_size), int(global_window_size)
+            if wl < 0 or wg < 0:
+                raise ValueError("window sizes must be >= 0")
+            block_mask = _masks.window_block_mask(nqb, wl, wg)
+        row_ptr, col_idx, csr_strides = _masks.block_mask_to_csr(block_mask, q.device)
+        if row_ptr.shape[-1] - 1 < nqb:
+            raise ValueError("block mask covers %d query blocks, sequences need %d" % (row_ptr.shape[-1] - 1, nqb))
+    a = _lib.AttnSparseArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _dtype_tag(q)
+    _fill_qkvo(a, qv, kv, vv, ov, lv, packed)
+    a.cu_seqlens = _ptr(cu)
+    a.row_ptr, a.col_idx = _ptr(row_ptr), _ptr(col_idx)
+    a.row_ptr_stride_b, a.row_ptr_stride_h, a.col_idx_stride_b, a.col_idx_stride_h = csr_strides
+    a.batch = batch
+    a.heads_q, a.heads_kv, a.head_dim = Hq, kv.shape[2], D
+    a.max_seqlen = max_len
+    a.block_size = _masks.BLOCK
+    a.window_local, a.window_global = wl, wg
+    a.scale_log2 = scale
+    _lib.check(lib.mi_attn_fwd_blocksparse(C.byref(a), _stream()))
+    return o, lse
+
+
+def _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, return_lse,
+            block_idx=None, block_cnt=None, bi_strides=(0, 0), max_blocks=0, split_blocks=0,
+            window=(-1, -1)):
+    _require_gpu(q, k, v, cu_seq_lens, seq_lens)
+    lib = _lib.load()
+    q, k, v = _inner_contig(q), _inner_contig(k), _inner_contig(v)
+    B, Hq, D = q.shape
+    Hkv = k.shape[2]
+    if v.shape[-1] != D or k.shape[-1] != D:
+        raise ValueError("q, k and v must share head_dim")
+    o = torch.empty((B, Hq, D), device=q.device, dtype=q.dtype)
+    lse = torch.empty((B, Hq), device=q.device, dtype=torch.float32) if return_lse else None
+    a = _lib.DecodeArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _dtype_tag(q)
+    a.q, a.k, a.v, a.o, a.lse = _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse)
+    a.q_stride_b, a.q_stride_h = q.stride(0), q.stride(1)
+    a.k_stride_b, a.k_stride_s, a.k_stride_h = k.stride(0), k.stride(1), k.stride(2)
+    a.v_stride_b, a.v_stride_s, a.v_stride_h = v.stride(0), v.stride(1), v.stride(2)
+    a.o_stride_b, a.o_stride_h = o.stride(0), o.stride(1)
+    if seq_lens is not None:
+        seq_lens = seq_lens.to(torch.int32)
+        a.seq_lens, a.cu_seqlens = _ptr(seq_lens), None
+    else:
+        cu_seq_lens = cu_seq_lens.to(torch.int32)
+        a.seq_lens, a.cu_seqlens = None, _ptr(cu_seq_lens)
+    a.batch, a.heads_q, a.heads_kv, a.head_dim = B, Hq, Hkv, D
+    # k.shape[1] bounds every length, so no host sync is needed for the grid
+    a.max_seqlen = int(k.shape[1] if max_seq_len is None else min(max_seq_len, k.shape[1]))
+    a.scale_log2 = float(scale) * LOG2E
+    if block_idx is None:
+        a.split_tokens = int(split_tokens) if split_tokens else lib.mi_decode_choose_split_tokens(
+            B, Hkv, a.max_seqlen, _NUM_CUS)
+    else:
+        a.split_tokens = 64
+        a.block_idx, a.block_cnt = _ptr(block_idx), _ptr(block_cnt)
+        a.block_idx_stride_b, a.block_idx_stride_h = bi_strides
+        a.max_blocks, a.block_size, a.split_blocks = int(max_blocks), _masks.BLOCK, int(split_blocks)
+        a.window_local, a.window_global = window
+    nbytes = lib.mi_decode_workspace_bytes(C.byref(a))
+    if nbytes == 0:
+        raise _lib.MiAttnError(lib.mi_decode_validate(C.byref(a)), lib.mi_last_error().decode())
+    ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
+    a.workspace, a.workspace_bytes = _ptr(ws), nbytes
+    _lib.check(lib.mi_decode(C.byref(a), _stream()))
+    return (o, lse) if return_lse else o
+
+
+def flash_attention_decoding(q, k, v, cu_seq_lens, qk_scale=None, *, seq_lens=None, max_seq_len=None,
+                             split_tokens=None, return_lse=False):
+    """Single-query decoding, split-KV + LSE merge.
+
+    Contract of flash_attention_decoding in
+    flash_attn_triton/flash_attn_decoding.py:213-336: q [B,Hq,D]; k, v
+    [B,maxL,Hkv,D] (any strides, e.g. a transposed view of [B,Hkv,L,D]);
+    cu_seq_lens [B+1] supplies only the lengths (:46-48); `qk_scale` natural
+    base, default D^-0.5 (:236-237).  Returns o [B,Hq,D]; rows with length 0
+    are zero.  Extensions: `seq_lens` [B] instead of cu_seq_lens, `max_seq_len`
+    and `split_tokens` to size the launch, `return_lse` (base-2, [B,Hq]).
+    """
+    if (cu_seq_lens is None) == (seq_lens is None):
+        raise ValueError("give exactly one of cu_seq_lens / seq_lens")
+    scale = q.shape[-1] ** -0.5 if qk_scale is None else qk_scale
+    return _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, return_lse)
+
+
+def flash_attention_sparse_decoding(q, k, v, cu_seq_lens, global_window_size=64, local_window_size=64, *,
+                                    seq_lens=None, block_indices=None, block_counts=None, block_size=64,
+                                    include_last_block=True, split_blocks=None, return_lse=False):
+    """Sparse single-query decoding.
+
+    Window form — contract of flash_attention_sparse_decoding in
+    flash_attn_triton/flash_attn_decoding_sparse.py:222-365: attends the first
+    `global_window_size` tokens and the last `local_window_size` tokens of each
+    sequence (oracle :391-396); global_window_size must be 64, 128 or 256
+    (:249-253); scale is D^-0.5 (:246).
+    Block form — `block_indices` [B,Hkv,n] int32 (unique, ascending, each in
+    [0, ceil(len/64))) lists the 64-token blocks each kv-head attends, shared
+    by its query heads; `block_counts` [B,Hkv] optionally gives the number of
+    valid entries; with `include_last_block` the block holding the newest
+    token is added if absent.  Tokens >= len are masked.
+    """
+    if (cu_seq_lens is None) == (seq_lens is None):
+        raise ValueError("give exactly one of cu_seq_lens / seq_lens")
+    if block_size != _masks.BLOCK:
+        raise ValueError("block_size must be %d" % _masks.BLOCK)
+    B, Hq, D = q.shape
+    Hkv = k.shape[2]
+    lens = seq_lens if seq_lens is not None else (cu_seq_lens[1:] - cu_seq_lens[:-1])
+    lens = lens.to(torch.int32)
+    scale = D ** -0.5
+    if block_indices is None:
+        gw, lw = int(global_window_size), int(local_window_size)
+        assert gw in {64, 128, 256}, "global_window_size must be one of 64, 128, or 256, got %d" % gw
+        if lw < 0:
+            raise ValueError("local_window_size must be >= 0")
+        n_sink = gw // _masks.BLOCK
+        n_tail = (lw + _masks.BLOCK - 1) // _masks.BLOCK + 1
+        nblk = (lens + _masks.BLOCK - 1) // _masks.BLOCK                      # [B]
+        tail0 = torch.clamp(lens - lw, min=0) // _masks.BLOCK
+        tail0 = torch.maximum(tail0, torch.full_like(tail0, n_sink))           # sink blocks listed once
+        cand = torch.cat([
+            torch.arange(n_sink, device=q.device, dtype=torch.int32).expand(B, n_sink),
+            tail0[:, None] + torch.arange(n_tail, device=q.device, dtype=torch.int32)[None, :],
+        ], dim=1)                                                              # [B, cap]
+        valid = cand < nblk[:, None]
+        key = torch.where(valid, cand, torch.full_like(cand, 2 ** 30))
+        idx = torch.sort(key, dim=1).values.to(torch.int32).contiguous()
+        idx = torch.where(idx >= 2 ** 30, torch.zeros_like(idx), idx)
+        cnt = valid.sum(1).to(torch.int32)[:, None].expand(B, Hkv).contiguous()
+        cap = n_sink + n_tail
+        return _decode(q, k, v, None, lens, scale, None, None, return_lse, block_idx=idx, block_cnt=cnt,
+                       bi_strides=(cap, 0), max_blocks=cap,
+                       split_blocks=split_blocks or max(1, min(8, cap)), window=(lw, gw))
+    idx = block_indices.to(torch.int32)
+    if idx.dim() != 3 or idx.shape[0] != B or idx.shape[1] != Hkv:
+        raise ValueError("block_indices must be [B, Hkv, n]")
+    n = idx.shape[2]
+    cnt = block_counts.to(torch.int32) if block_counts is not None else torch.full(
+        (B, Hkv), n, device=q.device, dtype=torch.int32)
+    if include_last_block:
+        last = torch.clamp((lens - 1) // _masks.BLOCK, min=0)[:, None, None].expand(B, Hkv, 1)
+        slot = torch.arange(n, device=q.device)[None, None, :]
+        present = ((idx == last) & (slot < cnt[..., None])).any(-1)
+        idx = torch.cat([idx, last.to(torch.int32)], dim=2)
+        # put the extra entry right after the valid ones
+        idx = idx.scatter(2, cnt[..., None].to(torch.int64), last.to(torch.int32))
+        cnt = cnt + (~present).to(torch.int32)
+        n += 1
+    idx = idx.contiguous()
+    cnt = cnt.contiguous()
+    return _decode(q, k, v, None, lens, scale, None, None, return_lse, block_idx=idx, block_cnt=cnt,
+                   bi_strides=(Hkv * n, n), max_blocks=n, split_blocks=split_blocks or max(1, min(8, n)))
