@@ -1,0 +1,310 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention forward hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+Prints ONE JSON line.  The headline workload is the dense causal bf16 forward
+B=4, H=32, S=8192, D=128 ("dense_causal"); the other benchmark configurations
+(GQA decode at 32k KV, block-sparse forward, block-sparse decode) are measured
+in the same run and reported under "other_workloads", each with its own
+roofline object.  --workload picks a single one as the headline instead.
+
+A step is one pass of the path over one batch of synthetic inputs that are
+already resident in HBM.  `value` comes from wall-clock around K steps
+bracketed by device synchronisation; `roofline.achieved` comes from HIP events
+recorded on the launch stream around the same kernels (mi_time_launches).
+The CPU baseline is the reference's PyTorch attention math (oracle/) timed on
+this host's cores on a stated slice of the same workload.
+"""
+import argparse
+import ctypes as C
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+
+def _sync():
+    torch.cuda.synchronize()
+
+
+def _randn(shape, seed, device="cuda"):
+    """Seeded N(0,1) -> bf16.  Big tensors are drawn on the device in chunks
+    (parity tests use CPU-drawn inputs; here only the distribution matters)."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    out = torch.empty(shape, device=device, dtype=torch.bfloat16)
+    flat = out.view(-1)
+    step = 1 << 28
+    for s in range(0, flat.numel(), step):
+        n = min(step, flat.numel() - s)
+        flat[s:s + n] = torch.randn(n, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    return out
+
+
+def _time_steps(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    _sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    _sync()
+    return (time.perf_counter() - t0) / steps * 1e3   # ms per step
+
+
+def _event_ms(kind, args, steps, warmup):
+    """Average launch duration from HIP events on the current stream."""
+    from tritonops_amd import _lib
+    lib = _lib.load()
+    ms = C.c_float(0)
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(lib.mi_time_launches(kind, C.cast(C.byref(args), C.c_void_p), st, warmup, steps, C.byref(ms)))
+    return ms.value
+
+
+# ----------------------------------------------------------------------------
+# workloads: each returns dict(ms_per_step, kernel_ms, work, unit-specific...)
+# ----------------------------------------------------------------------------
+def _fwd_args(q, k, v, o, lse, causal):
+    """mi_attn_fwd_args for contiguous [B,H,S,D] tensors."""
+    from tritonops_amd import _lib
+    B, H, S, D = q.shape
+    a = _lib.AttnFwdArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _lib.MI_DTYPE_BF16
+    a.q, a.k, a.v, a.o, a.lse = (t.data_ptr() for t in (q, k, v, o, lse))
+    for n, t in (("q", q), ("k", k), ("v", v), ("o", o)):
+        setattr(a, n + "_stride_b", t.stride(0))
+        setattr(a, n + "_stride_h", t.stride(1))
+        setattr(a, n + "_stride_s", t.stride(2))
+    a.lse_stride_b, a.lse_stride_h, a.lse_stride_s = lse.stride(0), lse.stride(1), lse.stride(2)
+    a.cu_seqlens = None
+    a.batch, a.heads_q, a.heads_kv, a.max_seqlen, a.head_dim = B, H, k.shape[1], S, D
+    a.causal = 1 if causal else 0
+    a.scale_log2 = D ** -0.5 * 1.4426950408889634
+    return a
+
+
+def run_dense_causal(steps, warmup):
+    import tritonops_amd as ta
+    B, H, S, D = 4, 32, 8192, 128
+    q, k, v = (_randn((B, H, S, D), s) for s in (0, 1, 2))
+    fn = lambda: ta.flash_attention(q, k, v, causal=True, return_lse=True)
+    ms = _time_steps(fn, steps, warmup)
+    o = torch.empty_like(q)
+    lse = torch.empty((B, H, S), device="cuda", dtype=torch.float32)
+    kms = _event_ms(0, _fwd_args(q, k, v, o, lse, True), steps, warmup)
+    flop = 2.0 * B * H * S * (S + 1) * D            # 4*D per unmasked (q, k) pair
+    return {
+        "name": "dense_causal", "ms_per_step": ms, "kernel_ms": kms,
+        "metric": "attn_fwd_tflops", "unit": "TFLOP/s", "value": flop / (ms * 1e-3) / 1e12,
+        "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "kernel": "prefill_kernel<bf16,128,dense>"},
+        "config": {"workload": "dense causal flash-attention fwd bf16 B=4 H=32 S=8192 D=128, o bf16 + lse fp32",
+                   "flop_per_step": flop, "flop_reference_convention_4BHS2D": 4.0 * B * H * S * S * D},
+    }
+
+
+def run_decode(steps, warmup):
+    import tritonops_amd as ta
+    B, Hq, Hkv, L, D = 64, 32, 8, 32768, 128
+    lens = torch.randint(16384, L + 1, (B,), generator=torch.Generator().manual_seed(1), dtype=torch.int32)
+    lens_d = lens.cuda()
+    q = _randn((B, Hq, D), 0)
+    # two KV sets, alternated, so no step finds its KV in the 256 MB last-level cache
+    caches = [(_randn((B, Hkv, L, D), 10 + 2 * i), _randn((B, Hkv, L, D), 11 + 2 * i)) for i in range(2)]
+    state = {"i": 0}
+
+    def fn():
+        kc, vc = caches[state["i"] & 1]
+        state["i"] += 1
+        return ta.flash_attention_decoding(q, kc.transpose(1, 2), vc.transpose(1, 2), None, seq_lens=lens_d)
+    ms = _time_steps(fn, steps, warmup)
+    # event timing of the two kernels on one cache (8.6 GB >> cache, no reuse between launches)
+    from tritonops_amd import _lib
+    lib = _lib.load()
+    kc, vc = caches[0]
+    k, v = kc.transpose(1, 2), vc.transpose(1, 2)
+    o = torch.empty((B, Hq, D), device="cuda", dtype=torch.bfloat16)
+    a = _lib.DecodeArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _lib.MI_DTYPE_BF16
+    a.q, a.k, a.v, a.o, a.lse = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), None
+    a.q_stride_b, a.q_stride_h = q.stride(0), q.stride(1)
+    a.k_stride_b, a.k_stride_s, a.k_stride_h = k.stride(0), k.stride(1), k.stride(2)
+    a.v_stride_b, a.v_stride_s, a.v_stride_h = v.stride(0), v.stride(1), v.stride(2)
+    a.o_stride_b, a.o_stride_h = o.stride(0), o.stride(1)
+    a.seq_lens, a.cu_seqlens = lens_d.data_ptr(), None
+    a.batch, a.heads_q, a.heads_kv, a.max_seqlen, a.head_dim = B, Hq, Hkv, L, D
+    a.scale_log2 = D ** -0.5 * 1.4426950408889634
+    a.split_tokens = lib.mi_decode_choose_split_tokens(B, Hkv, L, 256)
+    nbytes = lib.mi_decode_workspace_bytes(C.byref(a))
+    ws = torch.empty(nbytes, device="cuda", dtype=torch.uint8)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), nbytes
+    k_split = _event_ms(3, a, steps, warmup)
+    k_merge = _event_ms(4, a, steps, warmup)
+    nbytes_alg = float(lens.sum().item()) * Hkv * 2 * D * 2 + B * Hq * D * 2 * 2
+    return {
+        "name": "gqa_decode", "ms_per_step": ms, "kernel_ms": k_split, "merge_kernel_ms": k_merge,
+        "metric": "decode_hbm_gbs", "unit": "GB/s", "value": nbytes_alg / (ms * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "achieved": nbytes_alg / (k_split * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "kernel": "decode_splitkv_kernel<bf16,128>"},
+        "config": {"workload": "GQA decode bf16 B=64 Hq=32 Hkv=8 KV<=32768 (lens U[16384,32768]) D=128, split-KV + LSE merge",
+                   "bytes_per_step": nbytes_alg, "split_tokens": int(a.split_tokens)},
+    }
+
+
+def run_block_sparse(steps, warmup):
+    import tritonops_amd as ta
+    from tritonops_amd import masks
+    B, H, S, D = 2, 16, 16384, 128
+    nb = S // 64
+    m = masks.synthetic_block_mask(nb, 8, 4, 0.10, seed=2)
+    live = int(m.sum())
+    row_ptr, col_idx, strides = masks.block_mask_to_csr(m, "cuda")
+    q, k, v = (_randn((B, H, S, D), s) for s in (0, 1, 2))
+    fn = lambda: ta.flash_attn_sparse_triton(q, k, v, None, row_ptr=row_ptr, col_idx=col_idx, csr_strides=strides)
+    ms = _time_steps(fn, steps, warmup)
+    flop = 4.0 * D * ((live - nb) * 64 * 64 + nb * 64 * 65 / 2) * B * H
+    return {
+        "name": "block_sparse", "ms_per_step": ms, "kernel_ms": ms,
+        "metric": "sparse_attn_fwd_tflops", "unit": "TFLOP/s", "value": flop / (ms * 1e-3) / 1e12,
+        "roofline": {"bound": "mfma", "achieved": flop / (ms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "kernel": "prefill_kernel<bf16,128,sparse>"},
+        "config": {"workload": "block-sparse causal fwd bf16 B=2 H=16 S=16384 D=128, 64x64 blocks, band 8 + 4 sink + 10%% (%d live blocks)" % live,
+                   "flop_per_step": flop},
+    }
+
+
+def run_sparse_decode(steps, warmup):
+    import tritonops_amd as ta
+    from tritonops_amd import masks
+    B, Hq, Hkv, L, D = 32, 32, 8, 131072, 128
+    g = torch.Generator().manual_seed(1)
+    lens = (L - torch.randint(0, 64, (B,), generator=g)).to(torch.int32)
+    idx = masks.synthetic_decode_blocks(B, Hkv, L // 64, 128, seed=2).cuda()
+    lens_d = lens.cuda()
+    q = _randn((B, Hq, D), 0)
+    kc, vc = _randn((B, Hkv, L, D), 1), _randn((B, Hkv, L, D), 2)
+    fn = lambda: ta.flash_attention_sparse_decoding(q, kc.transpose(1, 2), vc.transpose(1, 2), None,
+                                                    seq_lens=lens_d, block_indices=idx)
+    ms = _time_steps(fn, steps, warmup)
+    nbytes_alg = float(B * Hkv * 129 * 64 * D * 2 * 2)
+    return {
+        "name": "sparse_decode", "ms_per_step": ms, "kernel_ms": ms,
+        "metric": "sparse_decode_hbm_gbs", "unit": "GB/s", "value": nbytes_alg / (ms * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "achieved": nbytes_alg / (ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "kernel": "decode_splitkv_kernel<bf16,128> (block list)"},
+        "config": {"workload": "block-sparse decode bf16 B=32 Hq=32 Hkv=8 KV=131072 D=128, top-128 of 64-token blocks + last block",
+                   "bytes_per_step": nbytes_alg, "note": "kernel_ms here is wall time of both passes plus the index preparation"},
+    }
+
+
+WORKLOADS = {
+    "dense_causal": run_dense_causal,
+    "gqa_decode": run_decode,
+    "block_sparse": run_block_sparse,
+    "sparse_decode": run_sparse_decode,
+}
+
+
+# ----------------------------------------------------------------------------
+# CPU baseline: the reference's PyTorch math on this host, bounded slice
+# ----------------------------------------------------------------------------
+def cpu_baseline(name):
+    from oracle import attention_oracle as orc
+    threads = torch.get_num_threads()
+    g = torch.Generator().manual_seed(0)
+
+    def med(fn, reps=3):
+        fn()
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return sorted(ts)[len(ts) // 2]
+
+    if name == "dense_causal":
+        B, H, S, D = 1, 2, 4096, 128
+        q, k, v = (torch.randn((B, H, S, D), generator=g).to(torch.bfloat16) for _ in range(3))
+        t = med(lambda: orc.causal_attention(q, k, v))
+        flop = 2.0 * B * H * S * (S + 1) * D
+        return {"value": flop / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "sample": "torch-CPU bf16 causal softmax(qk^T/sqrt(d))v (tutorial/4.4 oracle) on B=1 H=2 S=4096 D=128, "
+                          "median of 3; same algorithmic-FLOP formula as the GPU figure",
+                "seconds": t}
+    if name == "gqa_decode":
+        B, Hq, Hkv, L, D = 2, 32, 8, 32768, 128
+        lens = torch.randint(16384, L + 1, (B,), generator=g, dtype=torch.int32)
+        q = torch.randn((B, Hq, D), generator=g).to(torch.bfloat16)
+        k, v = (torch.randn((B, L, Hkv, D), generator=g).to(torch.bfloat16) for _ in range(2))
+        t = med(lambda: orc.flash_attn_decoding_torch(q, k, v, lens))
+        nb = float(lens.sum()) * Hkv * 2 * D * 2
+        return {"value": nb / t / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+                "sample": "torch-CPU bf16 decode oracle (flash_attn_decoding.py:339-368) on B=2 of the same shape, median of 3",
+                "seconds": t}
+    return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="all", choices=["all"] + list(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the attention path shards over batch and "
+                 "heads without communication); run with --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    from tritonops_amd import _lib
+    _lib.load()   # fail loudly when the HIP library is missing
+
+    names = list(WORKLOADS) if a.workload == "all" else [a.workload]
+    results = []
+    for n in names:
+        r = WORKLOADS[n](a.steps, a.warmup)
+        rf = r["roofline"]
+        rf["frac"] = rf["achieved"] / rf["peak"]
+        rf["traffic"] = None
+        results.append(r)
+        torch.cuda.empty_cache()
+    head = results[0]
+    out = {
+        "metric": head["metric"], "value": head["value"], "unit": head["unit"],
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic N(0,1) inputs drawn from a seed, resident in HBM",
+        "config": head["config"], "roofline": head["roofline"], "kernel_ms": head["kernel_ms"],
+        "device": torch.cuda.get_device_name(0),
+    }
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(head["name"])
+        if out["cpu_baseline"] is not None:
+            out["cpu_baseline"]["host_cpus"] = os.cpu_count()
+    if len(results) > 1:
+        out["other_workloads"] = [
+            {k: r[k] for k in ("name", "metric", "value", "unit", "ms_per_step", "kernel_ms", "roofline", "config")}
+            for r in results[1:]]
+        if not a.no_cpu_baseline:
+            for r in out["other_workloads"]:
+                cb = cpu_baseline(r["name"])
+                if cb is not None:
+                    r["cpu_baseline"] = cb
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

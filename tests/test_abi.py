@@ -1,0 +1,208 @@
+"""CPU-only checks of the C ABI: the library loads, exports every symbol that
+include/mi_attn.h declares, the ctypes structs match the C layout, and every
+validation error is reported before anything touches a device."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import pytest
+
+from tritonops_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mi_attn.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.load()
+
+
+def test_every_declared_symbol_is_exported(lib):
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = set(re.findall(r"\b(mi_[a-z_0-9]+)\s*\(", text))
+    assert declared, "no prototypes found in the header"
+    assert declared == set(_lib.EXPORTS), "ctypes table and header disagree: %s" % (declared ^ set(_lib.EXPORTS))
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.mi_abi_version() == 1
+
+
+def test_struct_layout_matches_the_c_compiler(tmp_path):
+    src = tmp_path / "sz.c"
+    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "mi_attn.h"\nint main(){printf("%zu %zu %zu %zu %zu %zu\\n",'
+                   "sizeof(mi_attn_fwd_args),sizeof(mi_attn_sparse_args),sizeof(mi_decode_args),"
+                   "offsetof(mi_attn_fwd_args,scale_log2),offsetof(mi_attn_sparse_args,scale_log2),"
+                   "offsetof(mi_decode_args,window_global));return 0;}\n")
+    exe = tmp_path / "sz"
+    subprocess.check_call(["gcc", "-std=c99", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
+    got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
+    want = [C.sizeof(_lib.AttnFwdArgs), C.sizeof(_lib.AttnSparseArgs), C.sizeof(_lib.DecodeArgs),
+            _lib.AttnFwdArgs.scale_log2.offset, _lib.AttnSparseArgs.scale_log2.offset,
+            _lib.DecodeArgs.window_global.offset]
+    assert got == want
+
+
+def _good_fwd():
+    a = _lib.AttnFwdArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = 0
+    a.q = a.k = a.v = a.o = 0x1000
+    for n in "qkvo":
+        setattr(a, n + "_stride_s", 128 * 4)
+        setattr(a, n + "_stride_h", 128)
+        setattr(a, n + "_stride_b", 128 * 4 * 64)
+    a.batch, a.heads_q, a.heads_kv, a.max_seqlen, a.head_dim, a.causal = 2, 4, 2, 64, 128, 1
+    a.scale_log2 = 0.1275
+    return a
+
+
+def _err(lib):
+    return lib.mi_last_error().decode()
+
+
+def test_fwd_validation(lib):
+    a = _good_fwd()
+    assert lib.mi_attn_fwd_validate(C.byref(a)) == 0
+    cases = [
+        (lambda a: setattr(a, "struct_size", 8), "MI_ERR_STRUCT_SIZE"),
+        (lambda a: setattr(a, "dtype", 7), "MI_ERR_DTYPE"),
+        (lambda a: setattr(a, "head_dim", 80), "MI_ERR_HEAD_DIM"),
+        (lambda a: setattr(a, "heads_kv", 3), "MI_ERR_GQA"),
+        (lambda a: setattr(a, "heads_q", 0), "MI_ERR_GQA"),
+        (lambda a: setattr(a, "batch", 0), "MI_ERR_SHAPE"),
+        (lambda a: setattr(a, "max_seqlen", -1), "MI_ERR_SHAPE"),
+        (lambda a: setattr(a, "causal", 2), "MI_ERR_SHAPE"),
+        (lambda a: setattr(a, "scale_log2", 0.0), "MI_ERR_SCALE"),
+        (lambda a: setattr(a, "scale_log2", float("nan")), "MI_ERR_SCALE"),
+        (lambda a: setattr(a, "q", None), "MI_ERR_NULL_POINTER"),
+        (lambda a: setattr(a, "k", 0x1004), "MI_ERR_ALIGNMENT"),
+        (lambda a: setattr(a, "v_stride_s", 100), "MI_ERR_STRIDE"),
+        (lambda a: setattr(a, "o_stride_b", 4), "MI_ERR_STRIDE"),
+    ]
+    for mutate, want in cases:
+        a = _good_fwd()
+        mutate(a)
+        rc = lib.mi_attn_fwd_validate(C.byref(a))
+        assert rc < 0 and lib.mi_status_name(rc).decode() == want == _lib.STATUS[rc], (want, rc)
+        assert _err(lib)
+        # the launch entry point refuses the same way, before any HIP call
+        assert lib.mi_attn_fwd(C.byref(a), None) == rc
+    assert lib.mi_attn_fwd_validate(None) == -1
+    # packed mode ignores batch strides
+    a = _good_fwd()
+    a.cu_seqlens = 0x2000
+    a.o_stride_b = 4
+    assert lib.mi_attn_fwd_validate(C.byref(a)) == 0
+
+
+def _good_sparse():
+    a = _lib.AttnSparseArgs()
+    a.struct_size = C.sizeof(a)
+    a.q = a.k = a.v = a.o = 0x1000
+    a.row_ptr = a.col_idx = 0x3000
+    for n in "qkvo":
+        setattr(a, n + "_stride_s", 256)
+        setattr(a, n + "_stride_h", 128)
+    a.batch, a.heads_q, a.heads_kv, a.max_seqlen, a.head_dim = 1, 2, 2, 640, 128
+    a.block_size, a.window_local, a.window_global = 64, -1, -1
+    a.scale_log2 = 0.1
+    return a
+
+
+def test_sparse_validation(lib):
+    assert lib.mi_attn_fwd_blocksparse_validate(C.byref(_good_sparse())) == 0
+    for mutate, want in [
+        (lambda a: setattr(a, "block_size", 128), "MI_ERR_SPARSE_LAYOUT"),
+        (lambda a: setattr(a, "row_ptr", None), "MI_ERR_NULL_POINTER"),
+        (lambda a: setattr(a, "window_local", 5), "MI_ERR_SPARSE_LAYOUT"),
+        (lambda a: setattr(a, "col_idx_stride_h", -1), "MI_ERR_SPARSE_LAYOUT"),
+        (lambda a: setattr(a, "head_dim", 256), "MI_ERR_HEAD_DIM"),
+    ]:
+        a = _good_sparse()
+        mutate(a)
+        rc = lib.mi_attn_fwd_blocksparse_validate(C.byref(a))
+        assert lib.mi_status_name(rc).decode() == want
+        assert lib.mi_attn_fwd_blocksparse(C.byref(a), None) == rc
+
+
+def _good_decode():
+    a = _lib.DecodeArgs()
+    a.struct_size = C.sizeof(a)
+    a.q = a.k = a.v = a.o = 0x1000
+    a.seq_lens = 0x2000
+    a.q_stride_b, a.q_stride_h = 32 * 128, 128
+    a.k_stride_b, a.k_stride_s, a.k_stride_h = 8 * 4096 * 128, 128, 4096 * 128
+    a.v_stride_b, a.v_stride_s, a.v_stride_h = 8 * 4096 * 128, 128, 4096 * 128
+    a.o_stride_b, a.o_stride_h = 32 * 128, 128
+    a.batch, a.heads_q, a.heads_kv, a.max_seqlen, a.head_dim = 4, 32, 8, 4096, 128
+    a.scale_log2 = 0.1
+    a.split_tokens = 512
+    a.workspace, a.workspace_bytes = 0x4000, 1 << 30
+    return a
+
+
+def test_decode_geometry_and_validation(lib):
+    a = _good_decode()
+    assert lib.mi_decode_num_splits(C.byref(a)) == 8
+    assert lib.mi_decode_workspace_bytes(C.byref(a)) == 4 * 32 * 8 * 129 * 4
+    assert lib.mi_decode_validate(C.byref(a)) == 0
+    for mutate, want in [
+        (lambda a: setattr(a, "split_tokens", 100), "MI_ERR_WORKSPACE"),
+        (lambda a: setattr(a, "workspace_bytes", 16), "MI_ERR_WORKSPACE"),
+        (lambda a: setattr(a, "workspace", None), "MI_ERR_NULL_POINTER"),
+        (lambda a: setattr(a, "cu_seqlens", 0x2000), "MI_ERR_NULL_POINTER"),     # both given
+        (lambda a: setattr(a, "seq_lens", None), "MI_ERR_NULL_POINTER"),         # none given
+        (lambda a: setattr(a, "heads_kv", 0), "MI_ERR_GQA"),
+        (lambda a: (setattr(a, "heads_q", 66), setattr(a, "heads_kv", 2)), "MI_ERR_GQA"),   # 33 per kv head
+        (lambda a: setattr(a, "k_stride_s", 12), "MI_ERR_STRIDE"),
+        (lambda a: setattr(a, "head_dim", 32), "MI_ERR_HEAD_DIM"),
+    ]:
+        a = _good_decode()
+        mutate(a)
+        rc = lib.mi_decode_validate(C.byref(a))
+        assert lib.mi_status_name(rc).decode() == want, (want, rc, _err(lib))
+        assert lib.mi_decode(C.byref(a), None) == rc
+    # sparse form
+    a = _good_decode()
+    a.block_idx = 0x5000
+    a.max_blocks, a.block_size, a.split_blocks = 129, 64, 8
+    a.window_local = a.window_global = -1
+    assert lib.mi_decode_num_splits(C.byref(a)) == 17
+    assert lib.mi_decode_validate(C.byref(a)) == 0
+    a.block_size = 32
+    assert lib.mi_status_name(lib.mi_decode_validate(C.byref(a))).decode() == "MI_ERR_SPARSE_LAYOUT"
+
+
+def test_split_heuristic(lib):
+    f = lib.mi_decode_choose_split_tokens
+    for args in [(64, 8, 32768, 256), (1, 1, 100, 256), (1, 8, 131072, 256), (512, 8, 4096, 256), (0, 0, 0, 0)]:
+        t = f(*args)
+        assert t % 64 == 0 and 64 <= t <= 4096
+    assert f(64, 8, 32768, 256) <= 4096
+    assert f(1, 1, 1 << 20, 256) == 256          # one sequence: as many chunks as allowed
+    assert f(4096, 8, 4096, 256) == 4096         # plenty of sequences: one chunk each
+
+
+def test_time_launches_rejects_bad_arguments(lib):
+    ms = C.c_float()
+    assert lib.mi_time_launches(0, None, None, 0, 1, C.byref(ms)) == -1
+    a = _good_fwd()
+    assert lib.mi_time_launches(9, C.cast(C.byref(a), C.c_void_p), None, 0, 1, C.byref(ms)) == -6
+    a.head_dim = 5
+    assert lib.mi_time_launches(0, C.cast(C.byref(a), C.c_void_p), None, 1, 1, C.byref(ms)) == -4
+
+
+def test_python_wrappers_refuse_cpu_tensors():
+    import torch
+
+    import tritonops_amd as ta
+
+    q = torch.zeros(1, 4, 2, 64, dtype=torch.bfloat16)
+    cu = torch.tensor([0, 4], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ta.flash_attention(q, q, q, cu)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ta.flash_attention_decoding(q[0], q, q, cu)
