@@ -28,13 +28,14 @@ template <typename T, int D>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2)))
 decode_splitkv_kernel(const DecodeParams p) {
   using G = RowGeom<D>;
-  constexpr int TILEB = kDecTile * G::ROWB;
+  constexpr int KTILEB = kDecTile * G::KROWB;
+  constexpr int VTILEB = kDecTile * G::VROWB;
   constexpr int NCHUNK = kDecTile * G::NCH;
   constexpr int LOADS = (NCHUNK + 63) / 64;
 
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * TILEB];
+  __shared__ __attribute__((aligned(16))) unsigned char smem[KTILEB + VTILEB];
   unsigned char* sK = smem;
-  unsigned char* sV = smem + TILEB;
+  unsigned char* sV = smem + KTILEB;
 
   const int lane = threadIdx.x;
   const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;

@@ -20,12 +20,14 @@ namespace mi {
 namespace {
 
 template <typename T, int D, int NW, bool SPARSE>
-__global__ void __launch_bounds__(NW * 64)
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2)))
 prefill_kernel(const PrefillParams p) {
   using G = RowGeom<D>;
   constexpr int BM = 32 * NW;
   constexpr int NT = 64 * NW;
-  constexpr int TILEB = kTileN * G::ROWB;
+  constexpr int KTILEB = kTileN * G::KROWB;
+  constexpr int VTILEB = kTileN * G::VROWB;
+  constexpr int STAGEB = KTILEB + VTILEB;
   constexpr int NCHUNK = kTileN * G::NCH;            // 16-byte chunks per tile
   constexpr int LOADS = (NCHUNK + NT - 1) / NT;      // per thread, per tensor
   constexpr int OROWB = D * 2 + 16;                  // epilogue staging row
@@ -133,8 +135,8 @@ prefill_kernel(const PrefillParams p) {
     }
   };
   auto lstore = [&](int stage) {
-    unsigned char* sK = smem + stage * 2 * TILEB;
-    unsigned char* sV = sK + TILEB;
+    unsigned char* sK = smem + stage * STAGEB;
+    unsigned char* sV = sK + KTILEB;
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       const int idx = tid + i * NT;
@@ -150,6 +152,10 @@ prefill_kernel(const PrefillParams p) {
     gload(SPARSE ? cols[0] : 0);
     lstore(0);
   }
+  // Drain every outstanding global load (the Q fragments) here, so that inside
+  // the loop the only loads in flight are the next tile's and no MFMA has to
+  // wait on a vector-memory counter.  s_waitcnt vmcnt(0) expcnt(7) lgkmcnt(15).
+  __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();
 
   for (int it = 0; it < n_tiles; ++it) {
@@ -171,8 +177,8 @@ prefill_kernel(const PrefillParams p) {
         if (SPARSE && wl >= 0) ok = ok && ((qrow - key < wl) || (key < wg));
         return ok;
       };
-      const unsigned char* sK = smem + (it & 1) * 2 * TILEB;
-      compute_tile<T, D, 2>(sK, sK + TILEB, lc, Qf, O, m, l, p.scale, need_mask, allowed);
+      const unsigned char* sK = smem + (it & 1) * STAGEB;
+      compute_tile<T, D, 2>(sK, sK + KTILEB, lc, Qf, O, m, l, p.scale, need_mask, allowed);
     }
     if (more) lstore((it + 1) & 1);
     __syncthreads();
@@ -210,7 +216,7 @@ prefill_kernel(const PrefillParams p) {
 
 template <int D, int NW>
 constexpr size_t prefill_lds_bytes() {
-  const size_t pipe = 2 * 2 * kTileN * RowGeom<D>::ROWB;
+  const size_t pipe = 2 * kTileN * (RowGeom<D>::KROWB + RowGeom<D>::VROWB);
   const size_t epi = (size_t)NW * 32 * (D * 2 + 16);
   return pipe > epi ? pipe : epi;
 }

@@ -15,10 +15,12 @@
 // accumulator registers feeding one PV MFMA are 8 CONSECUTIVE keys; V^T then
 // comes out of a row-major V tile with two ds_read_b64_tr_b16 per operand.
 //
-// LDS tile layout: row-major [key][head_dim padded to a power of two], 16-byte
-// chunks XOR-swizzled per row (no padding bytes), different swizzles for K
-// (read one 16 B chunk per lane, 32 different rows) and V (transposing reads,
-// 4 rows x 32 B per 16 lanes).
+// LDS tile layout: row-major [key][head_dim], rows padded so that the access
+// patterns below are bank-conflict free and every fragment address is a
+// per-lane base plus a compile-time immediate: K rows carry 16 pad bytes (a
+// fragment read takes one 16 B chunk from 16 consecutive rows per quarter
+// wave), V rows 64 pad bytes (a transposing read takes 64 B from each of 4
+// consecutive rows per half wave).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -69,23 +71,12 @@ template <int D>
 struct RowGeom {
   static_assert(D == 64 || D == 96 || D == 128, "head_dim");
   static constexpr int DP = (D == 64) ? 64 : 128;  // padded row, elements
-  static constexpr int ROWB = DP * 2;              // LDS bytes per row
+  static constexpr int KROWB = DP * 2 + 16;        // LDS bytes per K row
+  static constexpr int VROWB = DP * 2 + 64;        // LDS bytes per V row
   static constexpr int NCH = D / 8;                // real 16-byte chunks per row
   static constexpr int KSTEPS = D / 16;            // QK^T MFMA steps (k = 16)
   static constexpr int NDB = D / 32;               // 32-row blocks of O^T
 };
-
-// 16-byte-chunk swizzles.  K: a fragment read touches 32 rows at one logical
-// chunk.  V: a transposing read touches rows r..r+3 and r+8..r+11 at four
-// neighbouring chunks.
-template <int DP>
-__device__ __forceinline__ int swz_k(int row) {
-  return DP == 128 ? (row & 15) : ((row >> 1) & 7);
-}
-template <int DP>
-__device__ __forceinline__ int swz_v(int row) {
-  return DP == 128 ? (((row & 3) << 2) | ((row >> 2) & 3)) : (((row >> 1) & 1) << 2);
-}
 
 // Accumulator row rho of the 32x32 MFMA (rho = 8*(reg/4) + 4*(lane/32) + reg%4)
 // is fed from key key_perm(rho), which makes register r of lane-half h hold
@@ -120,36 +111,32 @@ __device__ __forceinline__ float sum_with_other_half(float x) {
 // Per-lane constants of the fragment addressing, computed once per kernel.
 template <int D>
 struct LaneCtx {
-  int lq;       // query column of this lane (lane % 32)
-  int lh;       // lane half (lane / 32)
-  int k_row;    // permuted K row inside a 32-key block
-  int k_swz;    // swizzle of that row (same for every 32-key block)
-  int v_row;    // first V row of the transposing read, relative to 16*kk
-  int v_chunk;  // logical chunk relative to 4*db
-  int v_sub;    // byte offset inside the chunk (0 / 8)
+  int lq;     // query column of this lane (lane % 32)
+  int lh;     // lane half (lane / 32)
+  int k_off;  // byte offset of this lane's K fragment inside a 32-key block, chunk 0
+  int v_off;  // byte offset of this lane's V^T fragment for kk = 0, db = 0, first read
 
   __device__ __forceinline__ void init(int lane) {
     using G = RowGeom<D>;
     lq = lane & 31;
     lh = lane >> 5;
-    k_row = key_perm(lq);
-    k_swz = swz_k<G::DP>(k_row);  // row + 32*kb keeps the same low bits
-    v_row = 8 * lh + ((lane & 15) >> 2);
-    v_chunk = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
-    v_sub = (lane & 1) * 8;
+    k_off = key_perm(lq) * G::KROWB + lh * 16;
+    // transposing read: lane j of a 16-lane group addresses row j/4, 8 bytes at
+    // element 4*(j%4) of the group's 16 columns; groups 0/1 (2/3) are the two
+    // column halves of lane half 0 (1), which starts 8 rows further down.
+    v_off = (8 * lh + ((lane & 15) >> 2)) * G::VROWB + (2 * ((lane >> 4) & 1) + ((lane & 3) >> 1)) * 16 +
+            (lane & 1) * 8;
   }
 };
 
-// Store one 16-byte chunk of a K / V row into its swizzled LDS slot.
+// Store one 16-byte chunk of a K / V row into its LDS slot.
 template <int D>
 __device__ __forceinline__ void lds_store_k(unsigned char* tile, int row, int ch, i32x4 val) {
-  using G = RowGeom<D>;
-  *reinterpret_cast<i32x4*>(tile + row * G::ROWB + ((ch ^ swz_k<G::DP>(row)) << 4)) = val;
+  *reinterpret_cast<i32x4*>(tile + row * RowGeom<D>::KROWB + (ch << 4)) = val;
 }
 template <int D>
 __device__ __forceinline__ void lds_store_v(unsigned char* tile, int row, int ch, i32x4 val) {
-  using G = RowGeom<D>;
-  *reinterpret_cast<i32x4*>(tile + row * G::ROWB + ((ch ^ swz_v<G::DP>(row)) << 4)) = val;
+  *reinterpret_cast<i32x4*>(tile + row * RowGeom<D>::VROWB + (ch << 4)) = val;
 }
 
 // A operand of O^T += V^T P^T for 16-key group kk and 32-wide d block db:
@@ -158,11 +145,8 @@ template <int D>
 __device__ __forceinline__ i32x4 load_vt_frag(const unsigned char* sV, const LaneCtx<D>& lc, int kk,
                                               int db) {
   using G = RowGeom<D>;
-  const int r0 = 16 * kk + lc.v_row;
-  const int r1 = r0 + 4;
-  const int ch = 4 * db + lc.v_chunk;
-  const unsigned char* a0 = sV + r0 * G::ROWB + ((ch ^ swz_v<G::DP>(r0)) << 4) + lc.v_sub;
-  const unsigned char* a1 = sV + r1 * G::ROWB + ((ch ^ swz_v<G::DP>(r1)) << 4) + lc.v_sub;
+  const unsigned char* a0 = sV + lc.v_off + (16 * kk) * G::VROWB + db * 64;
+  const unsigned char* a1 = a0 + 4 * G::VROWB;
   s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)a0);
   s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)a1);
   i32x2 l2 = __builtin_bit_cast(i32x2, lo);
@@ -171,11 +155,18 @@ __device__ __forceinline__ i32x4 load_vt_frag(const unsigned char* sV, const Lan
   return out;
 }
 
+// The running max may lag behind the true row max by up to this many binades
+// before the accumulators are rescaled: probabilities then reach 2^8 at most,
+// far inside the range of the 16-bit formats and of the fp32 sums, and the
+// final o = O / l and lse = m + log2(l) do not depend on which m was used.
+constexpr float kRescaleSlack = 8.0f;
+
 // One KV tile of NKB*32 keys against the wave's 32 queries.
 //   sK, sV : LDS tiles (row-major, swizzled) holding the keys of this tile
 //   Qf     : B operands of Q^T, chunk c covers d = 16c .. 16c+15
 //   O      : O^T accumulators, block db covers d = 32db .. 32db+31
-//   m      : running row max in the scaled base-2 domain (-inf at start)
+//   m      : reference max of the exponent, scaled base-2 domain (-inf at
+//            start); within kRescaleSlack of the true running max
 //   l      : this lane's share of the running row sum (the other half of the
 //            sum lives in lane l^32; add them at the end)
 //   allowed(key_in_tile) is consulted only when need_mask is true.
@@ -186,17 +177,36 @@ __device__ __forceinline__ void compute_tile(const unsigned char* sK, const unsi
                                              f32x16 (&O)[RowGeom<D>::NDB], float& m, float& l,
                                              float scale, bool need_mask, MaskF allowed) {
   using G = RowGeom<D>;
+  // S^T = K Q^T: NKB independent accumulator chains, stepped alternately, with
+  // the K fragments fetched kPrefetch steps ahead of the MFMA that uses them.
   f32x16 S[NKB];
+  {
+    constexpr int NSTEP = NKB * G::KSTEPS;
+    constexpr int kPrefetch = 4;
+    auto frag = [&](int s) -> i32x4 {
+      const int kb = s % NKB, c = s / NKB;
+      return *reinterpret_cast<const i32x4*>(sK + lc.k_off + kb * 32 * G::KROWB + 32 * c);
+    };
+    i32x4 kf[kPrefetch];
 #pragma unroll
-  for (int kb = 0; kb < NKB; ++kb) {
-    const unsigned char* rowp = sK + (kb * 32 + lc.k_row) * G::ROWB;
-    f32x16 acc = {0};
+    for (int s = 0; s < kPrefetch; ++s) kf[s] = frag(s);
 #pragma unroll
-    for (int c = 0; c < G::KSTEPS; ++c) {
-      const i32x4 kf = *reinterpret_cast<const i32x4*>(rowp + (((2 * c + lc.lh) ^ lc.k_swz) << 4));
-      acc = Elem<T>::mfma(kf, Qf[c], acc);
+    for (int kb = 0; kb < NKB; ++kb) S[kb] = (f32x16){0};
+#pragma unroll
+    for (int s = 0; s < NSTEP; ++s) {
+      S[s % NKB] = Elem<T>::mfma(kf[s % kPrefetch], Qf[s / NKB], S[s % NKB]);
+      if (s + kPrefetch < NSTEP) kf[s % kPrefetch] = frag(s + kPrefetch);
     }
-    S[kb] = acc;
+    // Pin that order for the instruction scheduler (it otherwise sinks every
+    // LDS read to just before its MFMA and exposes the LDS latency 16 times):
+    // kPrefetch reads, then one MFMA + one read per step, then the MFMA tail.
+    __builtin_amdgcn_sched_group_barrier(0x100, kPrefetch, 0);
+#pragma unroll
+    for (int s = 0; s < NSTEP - kPrefetch; ++s) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, kPrefetch, 0);
   }
 
   if (need_mask) {
@@ -216,10 +226,19 @@ __device__ __forceinline__ void compute_tile(const unsigned char* sK, const unsi
     for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S[kb][r]);
   mx = max_with_other_half(mx);
 
+  // Lazy rescale: keep exponentiating against the old max while the new one
+  // is at most kRescaleSlack above it (wave-uniform branch, rarely taken after
+  // the first tiles).
   const float m_new = fmaxf(m, mx * scale);
-  const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-  const float alpha = fast_exp2(m - m_safe);
-  m = m_new;
+  if (__builtin_amdgcn_ballot_w64(m_new > m + kRescaleSlack) != 0) {
+    // a lane whose keys were all masked so far has m = m_new = -inf: factor 0
+    const float alpha = fast_exp2(m - ((m_new == -INFINITY) ? 0.f : m_new));
+    l *= alpha;
+#pragma unroll
+    for (int db = 0; db < G::NDB; ++db) O[db] *= alpha;
+    m = m_new;
+  }
+  const float m_use = (m == -INFINITY) ? 0.f : m;  // nothing but masked keys so far
 
   uint32_t P[NKB][8];
   float rs = 0.f;
@@ -227,15 +246,12 @@ __device__ __forceinline__ void compute_tile(const unsigned char* sK, const unsi
   for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
     for (int r = 0; r < 16; r += 2) {
-      const float p0 = fast_exp2(fmaf(S[kb][r], scale, -m_safe));
-      const float p1 = fast_exp2(fmaf(S[kb][r + 1], scale, -m_safe));
+      const float p0 = fast_exp2(fmaf(S[kb][r], scale, -m_use));
+      const float p1 = fast_exp2(fmaf(S[kb][r + 1], scale, -m_use));
       rs += p0 + p1;
       P[kb][r >> 1] = Elem<T>::pack2(p0, p1);
     }
-  l = l * alpha + rs;
-
-#pragma unroll
-  for (int db = 0; db < G::NDB; ++db) O[db] *= alpha;
+  l += rs;
 
 #pragma unroll
   for (int kk = 0; kk < 2 * NKB; ++kk) {
