@@ -28,8 +28,9 @@ template <typename T, int D>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2)))
 decode_splitkv_kernel(const DecodeParams p) {
   using G = RowGeom<D>;
-  constexpr int KTILEB = kDecTile * G::KROWB;
-  constexpr int VTILEB = kDecTile * G::VROWB;
+  using F = PaddedFrags<D>;
+  constexpr int KTILEB = kDecTile * F::KROWB;
+  constexpr int VTILEB = kDecTile * F::VROWB;
   constexpr int NCHUNK = kDecTile * G::NCH;
   constexpr int LOADS = (NCHUNK + 63) / 64;
 
@@ -63,7 +64,7 @@ decode_splitkv_kernel(const DecodeParams p) {
   const T* kp = reinterpret_cast<const T*>(p.k) + b * p.k_sb + kvh * p.k_sh;
   const T* vp = reinterpret_cast<const T*>(p.v) + b * p.v_sb + kvh * p.v_sh;
 
-  LaneCtx<D> lc;
+  F lc;
   lc.init(lane);
 
   // Q^T operand: column lq is q-head kvh*gqa + lq, columns >= gqa are zero.
@@ -102,8 +103,8 @@ decode_splitkv_kernel(const DecodeParams p) {
       const int idx = lane + i * 64;
       if (NCHUNK % 64 == 0 || idx < NCHUNK) {
         const int row = idx / G::NCH, ch = idx % G::NCH;
-        lds_store_k<D>(sK, row, ch, kreg[i]);
-        lds_store_v<D>(sV, row, ch, vreg[i]);
+        F::store_k(sK, row, ch, kreg[i]);
+        F::store_v(sV, row, ch, vreg[i]);
       }
     }
   };

@@ -3,8 +3,10 @@
 //
 // Work decomposition: one workgroup = NW wavefronts = 32*NW consecutive query
 // rows of one (sequence, q-head); KV is walked in tiles of 64 keys that the
-// whole workgroup stages through LDS (double buffered, one barrier per tile);
-// each wavefront then runs compute_tile() on its own 32 rows.
+// whole workgroup brings into LDS with direct-to-LDS loads
+// (global_load_lds_dwordx4: no staging registers, no ds_write), double
+// buffered, one barrier per tile; each wavefront then runs compute_tile() on
+// its own 32 rows.
 //
 // Replaces flash_attn_fwd_kernel of flash_attn_triton/flash_attn_triton.py
 // :52-180 (dense) and flash_attn_triton/flash_attn_sparse_attn_triton.py
@@ -13,30 +15,39 @@
 // exp2+log2 pair per tile (:170); masks are built only for tiles that cross
 // the diagonal, the sequence end or a window edge (:148-154 builds one for
 // every tile); Q is read once (:155 re-reads it per tile).
+#include <type_traits>
+
 #include "kernels.h"
 #include "tile_core.h"
 
 namespace mi {
 namespace {
 
+typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(1))) const void glb_void;
+
+template <int V>
+using ic = std::integral_constant<int, V>;
+
 template <typename T, int D, int NW, bool SPARSE>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2)))
 prefill_kernel(const PrefillParams p) {
   using G = RowGeom<D>;
+  using F = SwizzledFrags<D>;
   constexpr int BM = 32 * NW;
-  constexpr int NT = 64 * NW;
-  constexpr int KTILEB = kTileN * G::KROWB;
-  constexpr int VTILEB = kTileN * G::VROWB;
-  constexpr int STAGEB = KTILEB + VTILEB;
-  constexpr int NCHUNK = kTileN * G::NCH;            // 16-byte chunks per tile
-  constexpr int LOADS = (NCHUNK + NT - 1) / NT;      // per thread, per tensor
-  constexpr int OROWB = D * 2 + 16;                  // epilogue staging row
+  constexpr int TILEB = kTileN * F::ROWB;   // one K or V tile
+  constexpr int STAGEB = 2 * TILEB;         // K tile then V tile
+  constexpr int RPI = 1024 / F::ROWB;       // tile rows filled by one direct-to-LDS instruction
+  constexpr int NINST = kTileN / RPI;       // such instructions per tensor per tile
+  constexpr int IPW = NINST / NW;           // ... per wavefront
+  static_assert(NINST % NW == 0, "tile rows must split evenly over the waves");
+  constexpr int OROWB = D * 2 + 16;         // epilogue staging row
 
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
   // ---- workgroup -> (sequence, head, q tile).  Consecutive workgroup ids are
   // dealt round-robin to the 8 XCDs, each with a private L2: give every XCD
@@ -88,10 +99,10 @@ prefill_kernel(const PrefillParams p) {
   const T* vp = reinterpret_cast<const T*>(p.v) + v_off + kvh * p.v_sh;
   T* op = reinterpret_cast<T*>(p.o) + o_off + h * p.o_sh;
 
-  LaneCtx<D> lc;
-  lc.init(lane);
+  F fr;
+  fr.init(lane);
   const int q0w = q0 + 32 * wave;
-  const int qrow = q0w + lc.lq;
+  const int qrow = q0w + fr.lq;
 
   // ---- tile list
   int n_tiles;
@@ -109,7 +120,7 @@ prefill_kernel(const PrefillParams p) {
   // ---- Q^T operands: lane (query lq, half lh) holds d = 16c + 8lh .. +7
   i32x4 Qf[G::KSTEPS];
   {
-    const T* qr = qp + (int64_t)min(qrow, len - 1) * p.q_ss + 8 * lc.lh;
+    const T* qr = qp + (int64_t)min(qrow, len - 1) * p.q_ss + 8 * fr.lh;
 #pragma unroll
     for (int c = 0; c < G::KSTEPS; ++c) Qf[c] = *reinterpret_cast<const i32x4*>(qr + 16 * c);
   }
@@ -119,49 +130,57 @@ prefill_kernel(const PrefillParams p) {
   for (int db = 0; db < G::NDB; ++db) O[db] = (f32x16){0};
   float m = -INFINITY, l = 0.f;
 
-  // ---- global -> register -> LDS staging of one K and one V tile
-  i32x4 kreg[LOADS], vreg[LOADS];
-  auto gload = [&](int col) {
+  // ---- direct-to-LDS tile loads.  Instruction t of this wave fills the 1 KiB
+  // of LDS that holds tile rows RPI*(wave + NW*t) .. +RPI-1: lane i's 16 bytes
+  // land in slot i of that KiB, i.e. row drow = i / SLOTS, slot dslot = i %
+  // SLOTS, which must receive logical chunk dslot ^ swz(row) of that row.
+  const int drow = lane / F::SLOTS, dslot = lane % F::SLOTS;
+  const int64_t k_rowb = p.k_ss * 2, v_rowb = p.v_ss * 2;  // bytes between keys
+  auto dma_tile = [&](int col, auto stage_c) {
+    constexpr int ST = decltype(stage_c)::value;
     const int k0 = col * kTileN;
+    const char* kt = reinterpret_cast<const char*>(kp) + k0 * k_rowb;
+    const char* vt = reinterpret_cast<const char*>(vp) + k0 * v_rowb;
+    unsigned char* sK = smem + ST * STAGEB;
+    unsigned char* sV = sK + TILEB;
+    if (k0 + kTileN <= len) {
+      // whole tile inside the sequence: uniform base + 32-bit lane offset
 #pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-      const int idx = tid + i * NT;
-      if (NCHUNK % NT == 0 || idx < NCHUNK) {
-        const int row = idx / G::NCH, ch = idx % G::NCH;
-        const int64_t kr = min(k0 + row, len - 1);  // clamp: masked later
-        kreg[i] = *reinterpret_cast<const i32x4*>(kp + kr * p.k_ss + ch * 8);
-        vreg[i] = *reinterpret_cast<const i32x4*>(vp + kr * p.v_ss + ch * 8);
+      for (int t = 0; t < IPW; ++t) {
+        const int inst = wave + NW * t;
+        const int r = RPI * inst + drow;
+        const int kc = dslot ^ F::swz_k(r), vc = dslot ^ F::swz_v(r);
+        const uint32_t kl = (uint32_t)drow * (uint32_t)k_rowb + (uint32_t)kc * 16u;
+        const uint32_t vl = (uint32_t)drow * (uint32_t)v_rowb + (uint32_t)vc * 16u;
+        if (D != 96 || kc < G::NCH)
+          __builtin_amdgcn_global_load_lds((glb_void*)(kt + (RPI * inst) * k_rowb + kl),
+                                           (lds_void*)(sK + inst * 1024), 16, 0, 0);
+        if (D != 96 || vc < G::NCH)
+          __builtin_amdgcn_global_load_lds((glb_void*)(vt + (RPI * inst) * v_rowb + vl),
+                                           (lds_void*)(sV + inst * 1024), 16, 0, 0);
       }
-    }
-  };
-  auto lstore = [&](int stage) {
-    unsigned char* sK = smem + stage * STAGEB;
-    unsigned char* sV = sK + KTILEB;
+    } else {
+      // rows past the sequence end re-read its last row (masked later)
 #pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-      const int idx = tid + i * NT;
-      if (NCHUNK % NT == 0 || idx < NCHUNK) {
-        const int row = idx / G::NCH, ch = idx % G::NCH;
-        lds_store_k<D>(sK, row, ch, kreg[i]);
-        lds_store_v<D>(sV, row, ch, vreg[i]);
+      for (int t = 0; t < IPW; ++t) {
+        const int inst = wave + NW * t;
+        const int r = RPI * inst + drow;
+        const int kc = dslot ^ F::swz_k(r), vc = dslot ^ F::swz_v(r);
+        const int64_t rr = min(k0 + r, len - 1) - k0;
+        if (D != 96 || kc < G::NCH)
+          __builtin_amdgcn_global_load_lds((glb_void*)(kt + rr * k_rowb + kc * 16), (lds_void*)(sK + inst * 1024),
+                                           16, 0, 0);
+        if (D != 96 || vc < G::NCH)
+          __builtin_amdgcn_global_load_lds((glb_void*)(vt + rr * v_rowb + vc * 16), (lds_void*)(sV + inst * 1024),
+                                           16, 0, 0);
       }
     }
   };
 
-  if (n_tiles > 0) {
-    gload(SPARSE ? cols[0] : 0);
-    lstore(0);
-  }
-  // Drain every outstanding global load (the Q fragments) here, so that inside
-  // the loop the only loads in flight are the next tile's and no MFMA has to
-  // wait on a vector-memory counter.  s_waitcnt vmcnt(0) expcnt(7) lgkmcnt(15).
-  __builtin_amdgcn_s_waitcnt(0x0F70);
-  __syncthreads();
-
-  for (int it = 0; it < n_tiles; ++it) {
+  auto step = [&](auto stage_c, int it) {
+    constexpr int ST = decltype(stage_c)::value;
     const int col = SPARSE ? cols[it] : it;
-    const bool more = it + 1 < n_tiles;
-    if (more) gload(SPARSE ? cols[it + 1] : it + 1);
+    if (it + 1 < n_tiles) dma_tile(SPARSE ? cols[it + 1] : it + 1, ic<ST ^ 1>{});
 
     const int k0 = col * kTileN;
     // whole tile above the diagonal for this wave: nothing to add
@@ -177,17 +196,30 @@ prefill_kernel(const PrefillParams p) {
         if (SPARSE && wl >= 0) ok = ok && ((qrow - key < wl) || (key < wg));
         return ok;
       };
-      const unsigned char* sK = smem + (it & 1) * STAGEB;
-      compute_tile<T, D, 2>(sK, sK + KTILEB, lc, Qf, O, m, l, p.scale, need_mask, allowed);
+      const unsigned char* sK = smem + ST * STAGEB;
+      compute_tile<T, D, 2>(sK, sK + TILEB, fr, Qf, O, m, l, p.scale, need_mask, allowed);
     }
-    if (more) lstore((it + 1) & 1);
+    // the next tile must have landed, and everyone must be done with this one
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0) expcnt(7) lgkmcnt(15)
     __syncthreads();
+  };
+
+  if (n_tiles > 0) dma_tile(SPARSE ? cols[0] : 0, ic<0>{});
+  // also drains the Q loads, so no MFMA in the loop waits on a memory counter
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
+
+  int it = 0;
+  for (; it + 1 < n_tiles; it += 2) {
+    step(ic<0>{}, it);
+    step(ic<1>{}, it + 1);
   }
+  if (it < n_tiles) step(ic<0>{}, it);
 
   // ---- epilogue: normalise, transpose through LDS, coalesced 16-byte stores
   const float l_tot = sum_with_other_half(l);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  if (p.lse && lc.lh == 0 && qrow < len) {
+  if (p.lse && fr.lh == 0 && qrow < len) {
     float* lp = p.lse + lse_off + h * p.lse_sh;
     lp[(int64_t)qrow * p.lse_ss] = l_tot > 0.f ? m + fast_log2(l_tot) : -INFINITY;
   }
@@ -196,11 +228,11 @@ prefill_kernel(const PrefillParams p) {
   for (int db = 0; db < G::NDB; ++db)
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      const int d = 32 * db + 8 * g + 4 * lc.lh;
+      const int d = 32 * db + 8 * g + 4 * fr.lh;
       i32x2 w;
       w[0] = (int)Elem<T>::pack2(O[db][4 * g] * inv, O[db][4 * g + 1] * inv);
       w[1] = (int)Elem<T>::pack2(O[db][4 * g + 2] * inv, O[db][4 * g + 3] * inv);
-      *reinterpret_cast<i32x2*>(stage + lc.lq * OROWB + d * 2) = w;
+      *reinterpret_cast<i32x2*>(stage + fr.lq * OROWB + d * 2) = w;
     }
   __syncthreads();
 #pragma unroll
@@ -216,7 +248,7 @@ prefill_kernel(const PrefillParams p) {
 
 template <int D, int NW>
 constexpr size_t prefill_lds_bytes() {
-  const size_t pipe = 2 * kTileN * (RowGeom<D>::KROWB + RowGeom<D>::VROWB);
+  const size_t pipe = 2 * 2 * kTileN * SwizzledFrags<D>::ROWB;
   const size_t epi = (size_t)NW * 32 * (D * 2 + 16);
   return pipe > epi ? pipe : epi;
 }

@@ -15,12 +15,18 @@
 // accumulator registers feeding one PV MFMA are 8 CONSECUTIVE keys; V^T then
 // comes out of a row-major V tile with two ds_read_b64_tr_b16 per operand.
 //
-// LDS tile layout: row-major [key][head_dim], rows padded so that the access
-// patterns below are bank-conflict free and every fragment address is a
-// per-lane base plus a compile-time immediate: K rows carry 16 pad bytes (a
-// fragment read takes one 16 B chunk from 16 consecutive rows per quarter
-// wave), V rows 64 pad bytes (a transposing read takes 64 B from each of 4
-// consecutive rows per half wave).
+// Two LDS tile layouts (both row-major [key][head_dim], both free of bank
+// conflicts for the two access patterns: a K fragment read takes one 16 B
+// chunk from 16 consecutive rows per quarter wave, a V transposing read takes
+// 64 B from each of 4 consecutive rows per half wave):
+//   PaddedFrags   - rows padded (K +16 B, V +64 B); every fragment address is a
+//                   lane base + immediate.  Filled with ds_write from registers
+//                   (decoding kernel).
+//   SwizzledFrags - unpadded rows, 16-byte chunks XOR-swizzled per row, so that
+//                   a global_load_lds_dwordx4 (64 lanes x 16 B, contiguous in
+//                   LDS) can fill 1 KiB of a tile directly; the XOR is applied
+//                   on the global-address side.  Fragment addresses are
+//                   precomputed per lane (prefill kernel).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -70,9 +76,7 @@ struct Elem<_Float16> {
 template <int D>
 struct RowGeom {
   static_assert(D == 64 || D == 96 || D == 128, "head_dim");
-  static constexpr int DP = (D == 64) ? 64 : 128;  // padded row, elements
-  static constexpr int KROWB = DP * 2 + 16;        // LDS bytes per K row
-  static constexpr int VROWB = DP * 2 + 64;        // LDS bytes per V row
+  static constexpr int DP = (D == 64) ? 64 : 128;  // row padded to a power of two, elements
   static constexpr int NCH = D / 8;                // real 16-byte chunks per row
   static constexpr int KSTEPS = D / 16;            // QK^T MFMA steps (k = 16)
   static constexpr int NDB = D / 32;               // 32-row blocks of O^T
@@ -89,14 +93,7 @@ __device__ __forceinline__ int key_perm(int rho) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
-// Value held by lane l^32.
-__device__ __forceinline__ float other_half(float x) {
-  const unsigned u = __builtin_bit_cast(unsigned, x);
-  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  // r[0]: both halves see the lower half's value; r[1]: the upper half's.
-  const unsigned lo = r[0], hi = r[1];
-  return __builtin_bit_cast(float, (threadIdx.x & 32) ? lo : hi);
-}
+// max / sum of x over lanes l and l^32.
 __device__ __forceinline__ float max_with_other_half(float x) {
   const unsigned u = __builtin_bit_cast(unsigned, x);
   auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
@@ -108,45 +105,7 @@ __device__ __forceinline__ float sum_with_other_half(float x) {
   return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
 }
 
-// Per-lane constants of the fragment addressing, computed once per kernel.
-template <int D>
-struct LaneCtx {
-  int lq;     // query column of this lane (lane % 32)
-  int lh;     // lane half (lane / 32)
-  int k_off;  // byte offset of this lane's K fragment inside a 32-key block, chunk 0
-  int v_off;  // byte offset of this lane's V^T fragment for kk = 0, db = 0, first read
-
-  __device__ __forceinline__ void init(int lane) {
-    using G = RowGeom<D>;
-    lq = lane & 31;
-    lh = lane >> 5;
-    k_off = key_perm(lq) * G::KROWB + lh * 16;
-    // transposing read: lane j of a 16-lane group addresses row j/4, 8 bytes at
-    // element 4*(j%4) of the group's 16 columns; groups 0/1 (2/3) are the two
-    // column halves of lane half 0 (1), which starts 8 rows further down.
-    v_off = (8 * lh + ((lane & 15) >> 2)) * G::VROWB + (2 * ((lane >> 4) & 1) + ((lane & 3) >> 1)) * 16 +
-            (lane & 1) * 8;
-  }
-};
-
-// Store one 16-byte chunk of a K / V row into its LDS slot.
-template <int D>
-__device__ __forceinline__ void lds_store_k(unsigned char* tile, int row, int ch, i32x4 val) {
-  *reinterpret_cast<i32x4*>(tile + row * RowGeom<D>::KROWB + (ch << 4)) = val;
-}
-template <int D>
-__device__ __forceinline__ void lds_store_v(unsigned char* tile, int row, int ch, i32x4 val) {
-  *reinterpret_cast<i32x4*>(tile + row * RowGeom<D>::VROWB + (ch << 4)) = val;
-}
-
-// A operand of O^T += V^T P^T for 16-key group kk and 32-wide d block db:
-// lane (d = 32*db + lane%32) receives V[16*kk + 8*(lane/32) + 0..7][d].
-template <int D>
-__device__ __forceinline__ i32x4 load_vt_frag(const unsigned char* sV, const LaneCtx<D>& lc, int kk,
-                                              int db) {
-  using G = RowGeom<D>;
-  const unsigned char* a0 = sV + lc.v_off + (16 * kk) * G::VROWB + db * 64;
-  const unsigned char* a1 = a0 + 4 * G::VROWB;
+__device__ __forceinline__ i32x4 read_tr_pair(const unsigned char* a0, const unsigned char* a1) {
   s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)a0);
   s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)a1);
   i32x2 l2 = __builtin_bit_cast(i32x2, lo);
@@ -155,66 +114,140 @@ __device__ __forceinline__ i32x4 load_vt_frag(const unsigned char* sV, const Lan
   return out;
 }
 
+// ---------------------------------------------------------------------------
+// Layout policy 1: padded rows.
+template <int D>
+struct PaddedFrags {
+  using G = RowGeom<D>;
+  static constexpr int KROWB = G::DP * 2 + 16;
+  static constexpr int VROWB = G::DP * 2 + 64;
+  int lq;     // query column of this lane (lane % 32)
+  int lh;     // lane half (lane / 32)
+  int k_off;  // byte offset of this lane's K fragment inside a 32-key block, chunk 0
+  int v_off;  // byte offset of this lane's V^T fragment for kk = 0, db = 0, first read
+
+  __device__ __forceinline__ void init(int lane) {
+    lq = lane & 31;
+    lh = lane >> 5;
+    k_off = key_perm(lq) * KROWB + lh * 16;
+    // transposing read: lane j of a 16-lane group addresses row j/4, 8 bytes at
+    // element 4*(j%4) of the group's 16 columns; groups 0/1 (2/3) are the two
+    // column halves of lane half 0 (1), which starts 8 rows further down.
+    v_off = (8 * lh + ((lane & 15) >> 2)) * VROWB + (2 * ((lane >> 4) & 1) + ((lane & 3) >> 1)) * 16 +
+            (lane & 1) * 8;
+  }
+  // A operand of S^T: K[32*kb + key_perm(lane%32)][16c + 8*(lane/32) .. +7]
+  __device__ __forceinline__ i32x4 load_k(const unsigned char* sK, int kb, int c) const {
+    return *reinterpret_cast<const i32x4*>(sK + k_off + kb * 32 * KROWB + 32 * c);
+  }
+  // A operand of O^T: V[16*kk + 8*(lane/32) + 0..7][32*db + lane%32]
+  __device__ __forceinline__ i32x4 load_v(const unsigned char* sV, int kk, int db) const {
+    const unsigned char* a0 = sV + v_off + (16 * kk) * VROWB + db * 64;
+    return read_tr_pair(a0, a0 + 4 * VROWB);
+  }
+  static __device__ __forceinline__ void store_k(unsigned char* tile, int row, int ch, i32x4 val) {
+    *reinterpret_cast<i32x4*>(tile + row * KROWB + (ch << 4)) = val;
+  }
+  static __device__ __forceinline__ void store_v(unsigned char* tile, int row, int ch, i32x4 val) {
+    *reinterpret_cast<i32x4*>(tile + row * VROWB + (ch << 4)) = val;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// Layout policy 2: XOR-swizzled 16-byte chunks, unpadded rows of DP*2 bytes.
+// LDS slot s of row r holds logical chunk s ^ swz(r).
+template <int D>
+struct SwizzledFrags {
+  using G = RowGeom<D>;
+  static constexpr int ROWB = G::DP * 2;
+  static constexpr int SLOTS = ROWB / 16;  // 16-byte slots per row
+  static __device__ __forceinline__ int swz_k(int row) {
+    return G::DP == 128 ? (row & 15) : ((row >> 1) & 7);
+  }
+  static __device__ __forceinline__ int swz_v(int row) {
+    return G::DP == 128 ? (((row & 3) << 2) | ((row >> 2) & 3)) : (((row >> 1) & 1) << 2);
+  }
+  int lq, lh;
+  uint32_t k_a[G::KSTEPS];  // byte offset of chunk step c inside a 32-key block
+  uint32_t v_a[G::NDB][2];  // byte offset of (d block, first/second read) inside a 16-key group
+
+  __device__ __forceinline__ void init(int lane) {
+    lq = lane & 31;
+    lh = lane >> 5;
+    const int krow = key_perm(lq);
+#pragma unroll
+    for (int c = 0; c < G::KSTEPS; ++c) k_a[c] = krow * ROWB + (((2 * c + lh) ^ swz_k(krow)) << 4);
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int r = 8 * lh + 4 * e + ((lane & 15) >> 2);
+#pragma unroll
+      for (int db = 0; db < G::NDB; ++db) {
+        const int ch = 4 * db + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+        v_a[db][e] = r * ROWB + ((ch ^ swz_v(r)) << 4) + (lane & 1) * 8;
+      }
+    }
+  }
+  // swz_k is invariant under row += 32, swz_v under row += 16
+  __device__ __forceinline__ i32x4 load_k(const unsigned char* sK, int kb, int c) const {
+    return *reinterpret_cast<const i32x4*>(sK + k_a[c] + kb * 32 * ROWB);
+  }
+  __device__ __forceinline__ i32x4 load_v(const unsigned char* sV, int kk, int db) const {
+    return read_tr_pair(sV + v_a[db][0] + kk * 16 * ROWB, sV + v_a[db][1] + kk * 16 * ROWB);
+  }
+};
+
 // The running max may lag behind the true row max by up to this many binades
 // before the accumulators are rescaled: probabilities then reach 2^8 at most,
 // far inside the range of the 16-bit formats and of the fp32 sums, and the
 // final o = O / l and lse = m + log2(l) do not depend on which m was used.
 constexpr float kRescaleSlack = 8.0f;
 
-// One KV tile of NKB*32 keys against the wave's 32 queries.
-//   sK, sV : LDS tiles (row-major, swizzled) holding the keys of this tile
-//   Qf     : B operands of Q^T, chunk c covers d = 16c .. 16c+15
-//   O      : O^T accumulators, block db covers d = 32db .. 32db+31
-//   m      : reference max of the exponent, scaled base-2 domain (-inf at
-//            start); within kRescaleSlack of the true running max
-//   l      : this lane's share of the running row sum (the other half of the
-//            sum lives in lane l^32; add them at the end)
-//   allowed(key_in_tile) is consulted only when need_mask is true.
-template <typename T, int D, int NKB, typename MaskF>
-__device__ __forceinline__ void compute_tile(const unsigned char* sK, const unsigned char* sV,
-                                             const LaneCtx<D>& lc,
-                                             const i32x4 (&Qf)[RowGeom<D>::KSTEPS],
-                                             f32x16 (&O)[RowGeom<D>::NDB], float& m, float& l,
-                                             float scale, bool need_mask, MaskF allowed) {
+// S^T = K Q^T for a tile of NKB 32-key blocks: NKB independent accumulator
+// chains stepped alternately, K fragments fetched kPrefetch steps ahead of the
+// MFMA that uses them.
+template <typename T, int D, int NKB, typename Frags>
+__device__ __forceinline__ void qk_scores(const unsigned char* sK, const Frags& fr,
+                                          const i32x4 (&Qf)[RowGeom<D>::KSTEPS], f32x16 (&S)[NKB]) {
   using G = RowGeom<D>;
-  // S^T = K Q^T: NKB independent accumulator chains, stepped alternately, with
-  // the K fragments fetched kPrefetch steps ahead of the MFMA that uses them.
-  f32x16 S[NKB];
-  {
-    constexpr int NSTEP = NKB * G::KSTEPS;
-    constexpr int kPrefetch = 4;
-    auto frag = [&](int s) -> i32x4 {
-      const int kb = s % NKB, c = s / NKB;
-      return *reinterpret_cast<const i32x4*>(sK + lc.k_off + kb * 32 * G::KROWB + 32 * c);
-    };
-    i32x4 kf[kPrefetch];
+  constexpr int NSTEP = NKB * G::KSTEPS;
+  constexpr int kPrefetch = 4;
+  i32x4 kf[kPrefetch];
 #pragma unroll
-    for (int s = 0; s < kPrefetch; ++s) kf[s] = frag(s);
+  for (int s = 0; s < kPrefetch; ++s) kf[s] = fr.load_k(sK, s % NKB, s / NKB);
 #pragma unroll
-    for (int kb = 0; kb < NKB; ++kb) S[kb] = (f32x16){0};
+  for (int kb = 0; kb < NKB; ++kb) S[kb] = (f32x16){0};
 #pragma unroll
-    for (int s = 0; s < NSTEP; ++s) {
-      S[s % NKB] = Elem<T>::mfma(kf[s % kPrefetch], Qf[s / NKB], S[s % NKB]);
-      if (s + kPrefetch < NSTEP) kf[s % kPrefetch] = frag(s + kPrefetch);
-    }
-    // Pin that order for the instruction scheduler (it otherwise sinks every
-    // LDS read to just before its MFMA and exposes the LDS latency 16 times):
-    // kPrefetch reads, then one MFMA + one read per step, then the MFMA tail.
-    __builtin_amdgcn_sched_group_barrier(0x100, kPrefetch, 0);
-#pragma unroll
-    for (int s = 0; s < NSTEP - kPrefetch; ++s) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, kPrefetch, 0);
+  for (int s = 0; s < NSTEP; ++s) {
+    S[s % NKB] = Elem<T>::mfma(kf[s % kPrefetch], Qf[s / NKB], S[s % NKB]);
+    if (s + kPrefetch < NSTEP) kf[s % kPrefetch] = fr.load_k(sK, (s + kPrefetch) % NKB, (s + kPrefetch) / NKB);
   }
+  // Pin that order for the instruction scheduler (it otherwise sinks every LDS
+  // read to just before its MFMA and exposes the LDS latency at every step):
+  // kPrefetch reads, then one MFMA + one read per step, then the MFMA tail.
+  __builtin_amdgcn_sched_group_barrier(0x100, kPrefetch, 0);
+#pragma unroll
+  for (int s = 0; s < NSTEP - kPrefetch; ++s) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+  }
+  __builtin_amdgcn_sched_group_barrier(0x008, kPrefetch, 0);
+}
 
+// Online-softmax step on the scores of one tile.  On return P holds the packed
+// 16-bit probabilities (P[kb][i] = keys 2i, 2i+1 of the lane's 16 keys in block
+// kb), l has this lane's share of the row sum added, and O / l / m have been
+// rescaled if the row max outgrew the slack.
+template <typename T, int D, int NKB, typename MaskF>
+__device__ __forceinline__ void softmax_tile(f32x16 (&S)[NKB], int lh, f32x16 (&O)[RowGeom<D>::NDB], float& m,
+                                             float& l, float scale, bool need_mask, MaskF allowed,
+                                             uint32_t (&P)[NKB][8]) {
+  using G = RowGeom<D>;
   if (need_mask) {
 #pragma unroll
     for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int key = kb * 32 + 16 * (r >> 3) + 8 * lc.lh + (r & 7);
+        const int key = kb * 32 + 16 * (r >> 3) + 8 * lh + (r & 7);
         if (!allowed(key)) S[kb][r] = -INFINITY;
       }
   }
@@ -240,7 +273,6 @@ __device__ __forceinline__ void compute_tile(const unsigned char* sK, const unsi
   }
   const float m_use = (m == -INFINITY) ? 0.f : m;  // nothing but masked keys so far
 
-  uint32_t P[NKB][8];
   float rs = 0.f;
 #pragma unroll
   for (int kb = 0; kb < NKB; ++kb)
@@ -252,17 +284,44 @@ __device__ __forceinline__ void compute_tile(const unsigned char* sK, const unsi
       P[kb][r >> 1] = Elem<T>::pack2(p0, p1);
     }
   l += rs;
+}
 
+// O^T += V^T P^T for one tile.
+template <typename T, int D, int NKB, typename Frags>
+__device__ __forceinline__ void pv_accumulate(const unsigned char* sV, const Frags& fr,
+                                              const uint32_t (&P)[NKB][8], f32x16 (&O)[RowGeom<D>::NDB]) {
+  using G = RowGeom<D>;
 #pragma unroll
   for (int kk = 0; kk < 2 * NKB; ++kk) {
     const int kb = kk >> 1, o4 = (kk & 1) * 4;
     const i32x4 pf = {(int)P[kb][o4], (int)P[kb][o4 + 1], (int)P[kb][o4 + 2], (int)P[kb][o4 + 3]};
 #pragma unroll
     for (int db = 0; db < G::NDB; ++db) {
-      const i32x4 vf = load_vt_frag<D>(sV, lc, kk, db);
+      const i32x4 vf = fr.load_v(sV, kk, db);
       O[db] = Elem<T>::mfma(vf, pf, O[db]);
     }
   }
+}
+
+// One KV tile of NKB*32 keys against the wave's 32 queries.
+//   sK, sV : LDS tiles holding the keys of this tile, in the layout of Frags
+//   Qf     : B operands of Q^T, chunk c covers d = 16c .. 16c+15
+//   O      : O^T accumulators, block db covers d = 32db .. 32db+31
+//   m      : reference max of the exponent, scaled base-2 domain (-inf at
+//            start); within kRescaleSlack of the true running max
+//   l      : this lane's share of the running row sum (the other half of the
+//            sum lives in lane l^32; add them at the end)
+//   allowed(key_in_tile) is consulted only when need_mask is true.
+template <typename T, int D, int NKB, typename Frags, typename MaskF>
+__device__ __forceinline__ void compute_tile(const unsigned char* sK, const unsigned char* sV,
+                                             const Frags& fr, const i32x4 (&Qf)[RowGeom<D>::KSTEPS],
+                                             f32x16 (&O)[RowGeom<D>::NDB], float& m, float& l,
+                                             float scale, bool need_mask, MaskF allowed) {
+  f32x16 S[NKB];
+  uint32_t P[NKB][8];
+  qk_scores<T, D, NKB>(sK, fr, Qf, S);
+  softmax_tile<T, D, NKB>(S, fr.lh, O, m, l, scale, need_mask, allowed, P);
+  pv_accumulate<T, D, NKB>(sV, fr, P, O);
 }
 
 }  // namespace mi
