@@ -58,7 +58,10 @@ int launch_decode_splitkv(const DecodeParams& p, int dtype, int head_dim, hipStr
 int launch_decode_merge(const DecodeParams& p, int dtype, int head_dim, hipStream_t s);
 
 // Query rows per workgroup of the two prefill kernels.
-constexpr int kDenseRows = 128;
+constexpr int kDenseRows = 256;
 constexpr int kSparseRows = 64;
+// LDS stages (KV tiles resident per workgroup) of the two prefill kernels.
+constexpr int kDenseStages = 3;
+constexpr int kSparseStages = 2;
 
 }  // namespace mi

@@ -29,14 +29,18 @@ typedef __attribute__((address_space(1))) const void glb_void;
 template <int V>
 using ic = std::integral_constant<int, V>;
 
-template <typename T, int D, int NW, bool SPARSE>
+// vmcnt(N) expcnt(7) lgkmcnt(15) for s_waitcnt on gfx9-family encodings
+constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
+
+// NW wavefronts per workgroup, NS LDS stages (tiles in flight + the one in use).
+template <typename T, int D, int NW, int NS, bool SPARSE>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2)))
 prefill_kernel(const PrefillParams p) {
   using G = RowGeom<D>;
   using F = SwizzledFrags<D>;
   constexpr int BM = 32 * NW;
   constexpr int TILEB = kTileN * F::ROWB;   // one K or V tile
-  constexpr int STAGEB = 2 * TILEB;         // K tile then V tile
+  constexpr int VBASE = NS * TILEB;         // LDS: NS K tiles, then NS V tiles
   constexpr int RPI = 1024 / F::ROWB;       // tile rows filled by one direct-to-LDS instruction
   constexpr int NINST = kTileN / RPI;       // such instructions per tensor per tile
   constexpr int IPW = NINST / NW;           // ... per wavefront
@@ -100,7 +104,7 @@ prefill_kernel(const PrefillParams p) {
   T* op = reinterpret_cast<T*>(p.o) + o_off + h * p.o_sh;
 
   F fr;
-  fr.init(lane);
+  fr.init(lane, VBASE);
   const int q0w = q0 + 32 * wave;
   const int qrow = q0w + fr.lq;
 
@@ -141,8 +145,8 @@ prefill_kernel(const PrefillParams p) {
     const int k0 = col * kTileN;
     const char* kt = reinterpret_cast<const char*>(kp) + k0 * k_rowb;
     const char* vt = reinterpret_cast<const char*>(vp) + k0 * v_rowb;
-    unsigned char* sK = smem + ST * STAGEB;
-    unsigned char* sV = sK + TILEB;
+    unsigned char* sK = smem + ST * TILEB;
+    unsigned char* sV = smem + VBASE + ST * TILEB;
     if (k0 + kTileN <= len) {
       // whole tile inside the sequence: uniform base + 32-bit lane offset
 #pragma unroll
@@ -180,7 +184,9 @@ prefill_kernel(const PrefillParams p) {
   auto step = [&](auto stage_c, int it) {
     constexpr int ST = decltype(stage_c)::value;
     const int col = SPARSE ? cols[it] : it;
-    if (it + 1 < n_tiles) dma_tile(SPARSE ? cols[it + 1] : it + 1, ic<ST ^ 1>{});
+    // refill the stage that was read in the previous iteration
+    const bool refill = it + NS - 1 < n_tiles;
+    if (refill) dma_tile(SPARSE ? cols[it + NS - 1] : it + NS - 1, ic<(ST + NS - 1) % NS>{});
 
     const int k0 = col * kTileN;
     // whole tile above the diagonal for this wave: nothing to add
@@ -196,25 +202,43 @@ prefill_kernel(const PrefillParams p) {
         if (SPARSE && wl >= 0) ok = ok && ((qrow - key < wl) || (key < wg));
         return ok;
       };
-      const unsigned char* sK = smem + ST * STAGEB;
-      compute_tile<T, D, 2>(sK, sK + TILEB, fr, Qf, O, m, l, p.scale, need_mask, allowed);
+      // V addresses carry VBASE inside the lane offsets (see fr.init)
+      compute_tile<T, D, 2>(smem + ST * TILEB, smem + ST * TILEB, fr, Qf, O, m, l, p.scale, need_mask, allowed);
     }
-    // the next tile must have landed, and everyone must be done with this one
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0) expcnt(7) lgkmcnt(15)
+    // The next tile must have landed and everyone must be done with this one.
+    // This wave's loads complete in order, so it is enough that at most the
+    // loads of the NS-2 younger tiles are still in flight (2*IPW each).
+    if (refill)
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * 2 * IPW));
+    else
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __syncthreads();
   };
 
-  if (n_tiles > 0) dma_tile(SPARSE ? cols[0] : 0, ic<0>{});
-  // also drains the Q loads, so no MFMA in the loop waits on a memory counter
-  __builtin_amdgcn_s_waitcnt(0x0F70);
+#pragma unroll
+  for (int s0 = 0; s0 < NS - 1; ++s0)
+    if (s0 < n_tiles) {
+      if (s0 == 0) dma_tile(SPARSE ? cols[0] : 0, ic<0>{});
+      if (s0 == 1) dma_tile(SPARSE ? cols[1] : 1, ic<1 % NS>{});
+      if (s0 == 2) dma_tile(SPARSE ? cols[2] : 2, ic<2 % NS>{});
+    }
+  // tile 0 (and the Q loads issued before it) must be complete
+  if (n_tiles >= NS - 1)
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * 2 * IPW));
+  else
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
   __syncthreads();
 
   int it = 0;
-  for (; it + 1 < n_tiles; it += 2) {
+  for (; it + NS <= n_tiles; it += NS) {
     step(ic<0>{}, it);
-    step(ic<1>{}, it + 1);
+    step(ic<1 % NS>{}, it + 1);
+    if (NS > 2) step(ic<2 % NS>{}, it + 2);
+    if (NS > 3) step(ic<3 % NS>{}, it + 3);
   }
-  if (it < n_tiles) step(ic<0>{}, it);
+  if (it < n_tiles) step(ic<0>{}, it++);
+  if (it < n_tiles) step(ic<1 % NS>{}, it++);
+  if (NS > 3 && it < n_tiles) step(ic<2 % NS>{}, it++);
 
   // ---- epilogue: normalise, transpose through LDS, coalesced 16-byte stores
   const float l_tot = sum_with_other_half(l);
@@ -246,17 +270,18 @@ prefill_kernel(const PrefillParams p) {
   }
 }
 
-template <int D, int NW>
+template <int D, int NW, int NS>
 constexpr size_t prefill_lds_bytes() {
-  const size_t pipe = 2 * 2 * kTileN * SwizzledFrags<D>::ROWB;
+  const size_t pipe = (size_t)NS * 2 * kTileN * SwizzledFrags<D>::ROWB;
   const size_t epi = (size_t)NW * 32 * (D * 2 + 16);
   return pipe > epi ? pipe : epi;
 }
 
 template <typename T, int D, int NW, bool SPARSE>
 int launch_one(const PrefillParams& p, hipStream_t s) {
-  auto kern = prefill_kernel<T, D, NW, SPARSE>;
-  constexpr size_t lds = prefill_lds_bytes<D, NW>();
+  constexpr int NS = SPARSE ? kSparseStages : kDenseStages;
+  auto kern = prefill_kernel<T, D, NW, NS, SPARSE>;
+  constexpr size_t lds = prefill_lds_bytes<D, NW, NS>();
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return (int)e;

@@ -171,7 +171,10 @@ struct SwizzledFrags {
   uint32_t k_a[G::KSTEPS];  // byte offset of chunk step c inside a 32-key block
   uint32_t v_a[G::NDB][2];  // byte offset of (d block, first/second read) inside a 16-key group
 
-  __device__ __forceinline__ void init(int lane) {
+  // v_bias is folded into the V fragment offsets: the V tiles may then live
+  // beyond the 64 KiB reach of a DS immediate while every read still is
+  // "lane register + immediate" relative to the K tile of the same stage.
+  __device__ __forceinline__ void init(int lane, int v_bias) {
     lq = lane & 31;
     lh = lane >> 5;
     const int krow = key_perm(lq);
@@ -183,7 +186,7 @@ struct SwizzledFrags {
 #pragma unroll
       for (int db = 0; db < G::NDB; ++db) {
         const int ch = 4 * db + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
-        v_a[db][e] = r * ROWB + ((ch ^ swz_v(r)) << 4) + (lane & 1) * 8;
+        v_a[db][e] = v_bias + r * ROWB + ((ch ^ swz_v(r)) << 4) + (lane & 1) * 8;
       }
     }
   }
