@@ -172,7 +172,9 @@ int mi_attn_fwd_blocksparse(const mi_attn_sparse_args *args, void *stream);
  *   block_idx[b*block_idx_stride_b + h*block_idx_stride_h + i],
  *   i < (block_cnt ? block_cnt[b*heads_kv + h] : max_blocks),
  * each `block_size` (64) tokens; indices must be unique and in range
- * [0, ceil(seq_len/block_size)); tokens >= seq_len are masked.  On top of the
+ * [0, ceil(seq_len/block_size)); tokens >= seq_len are masked.  With
+ * include_last_block the block of the newest token is attended as well; if it
+ * is also listed it still counts once.  On top of the
  * list an optional token window reproduces flash_attn_decoding_sparse.py
  * :391-396:  allowed(k) = k < window_global or k >= seq_len - window_local
  * (pass -1/-1 to disable).
@@ -207,6 +209,8 @@ typedef struct mi_decode_args {
   int32_t split_blocks;          /* sparse: listed blocks per workgroup        */
   int32_t window_local;          /* tokens, or -1                              */
   int32_t window_global;         /* tokens, or -1                              */
+  int32_t include_last_block;    /* 1: also attend the block holding token     */
+                                 /* seq_len-1 (listed or not, counted once)    */
 } mi_decode_args;
 
 /* Number of pass-1 chunks per sequence for these arguments (host only). */

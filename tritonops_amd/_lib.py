@@ -87,6 +87,7 @@ class DecodeArgs(C.Structure):
         ("block_idx_stride_b", _i64), ("block_idx_stride_h", _i64),
         ("max_blocks", _i32), ("block_size", _i32), ("split_blocks", _i32),
         ("window_local", _i32), ("window_global", _i32),
+        ("include_last_block", _i32),
     ]
 
 

@@ -76,7 +76,7 @@ void fill_prefill(const A* a, mi::PrefillParams& p, int rows_per_wg) {
 }
 
 int decode_splits(const mi_decode_args* a) {
-  if (a->block_idx) return (a->max_blocks + a->split_blocks - 1) / a->split_blocks;
+  if (a->block_idx) return (a->max_blocks + (a->include_last_block ? 1 : 0) + a->split_blocks - 1) / a->split_blocks;
   return (a->max_seqlen + a->split_tokens - 1) / a->split_tokens;
 }
 
@@ -99,6 +99,7 @@ void fill_decode(const mi_decode_args* a, mi::DecodeParams& p) {
   p.max_blocks = a->max_blocks; p.split_blocks = a->split_blocks;
   p.win_local = a->block_idx ? a->window_local : -1;
   p.win_global = a->block_idx ? a->window_global : -1;
+  p.add_last = (a->block_idx && a->include_last_block) ? 1 : 0;
   if (!a->block_idx) { p.max_blocks = 0; p.split_blocks = 1; }
 }
 
@@ -201,6 +202,8 @@ static int decode_validate_shape(const mi_decode_args* a) {
     return fail(MI_ERR_GQA, "at most 32 query heads per kv head (got %d)", a->heads_q / a->heads_kv);
   if (a->block_idx) {
     if (a->block_size != MI_ATTN_BLOCK) return fail(MI_ERR_SPARSE_LAYOUT, "block_size %d must be %d", a->block_size, MI_ATTN_BLOCK);
+    if (a->include_last_block != 0 && a->include_last_block != 1)
+      return fail(MI_ERR_SPARSE_LAYOUT, "include_last_block must be 0 or 1");
     if (a->max_blocks <= 0 || a->split_blocks <= 0)
       return fail(MI_ERR_SPARSE_LAYOUT, "max_blocks %d and split_blocks %d must be positive", a->max_blocks, a->split_blocks);
     if (a->block_idx_stride_b < 0 || a->block_idx_stride_h < 0)
@@ -229,13 +232,13 @@ size_t mi_decode_workspace_bytes(const mi_decode_args* a) {
 }
 
 int mi_decode_choose_split_tokens(int batch, int heads_kv, int max_seqlen, int num_cus) {
-  // One wavefront per (chunk, kv-head, sequence); aim for ~16 wavefronts per
+  // One wavefront per (chunk, kv-head, sequence); aim for ~32 wavefronts per
   // compute unit's worth of chunks so the tail is short, with chunks no shorter
   // than 256 tokens (partials stay < 2 % of the KV bytes) and no longer than 4096.
   if (batch <= 0 || heads_kv <= 0 || max_seqlen <= 0) return 64;
   if (num_cus <= 0) num_cus = 256;
   const long long units = (long long)batch * heads_kv;
-  const long long want = 16LL * num_cus;
+  const long long want = 32LL * num_cus;
   long long splits = (want + units - 1) / units;
   if (splits < 1) splits = 1;
   long long tokens = (max_seqlen + splits - 1) / splits;

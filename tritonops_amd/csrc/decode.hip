@@ -46,19 +46,30 @@ decode_splitkv_kernel(const DecodeParams p) {
 
   int n_tiles, t_begin = 0;
   const int32_t* blist = nullptr;
+  int n_listed = 0;  // listed entries that fall into this chunk
+  const int last_blk = (len - 1) / 64;
   if (sparse) {
     const int cnt = p.block_cnt ? min(p.block_cnt[b * p.hkv + kvh], p.max_blocks) : p.max_blocks;
+    const int total = cnt + p.add_last;  // the implicit last block sits behind the list
     const int b0 = split * p.split_blocks;
-    if (b0 >= cnt || len <= 0) return;
+    if (b0 >= total || len <= 0) return;
     blist = p.block_idx + b * p.bi_sb + kvh * p.bi_sh + b0;
-    n_tiles = 2 * min(cnt - b0, p.split_blocks);
+    n_tiles = 2 * min(total - b0, p.split_blocks);
+    n_listed = max(0, min(cnt - b0, p.split_blocks));
   } else {
     t_begin = split * p.split_tokens;
     if (t_begin >= len) return;
     n_tiles = (min(len, t_begin + p.split_tokens) - t_begin + kDecTile - 1) / kDecTile;
   }
+  // sparse: entry i/2 of the chunk; entries behind the listed ones are the
+  // implicit last block, and a LISTED last block is dropped when the implicit
+  // one exists (base -1 => the whole tile is masked)
   auto tile_base = [&](int i) -> int {
-    return sparse ? blist[i >> 1] * 64 + (i & 1) * kDecTile : t_begin + i * kDecTile;
+    if (!sparse) return t_begin + i * kDecTile;
+    const int e = i >> 1;
+    const int blk = e < n_listed ? blist[e] : last_blk;
+    if (p.add_last && e < n_listed && blk == last_blk) return -1;
+    return blk * 64 + (i & 1) * kDecTile;
   };
 
   const T* kp = reinterpret_cast<const T*>(p.k) + b * p.k_sb + kvh * p.k_sh;
@@ -116,11 +127,11 @@ decode_splitkv_kernel(const DecodeParams p) {
     const int base = tile_base(it);
     const bool more = it + 1 < n_tiles;
     if (more) gload(tile_base(it + 1));
-    bool need_mask = base + kDecTile > len;
+    bool need_mask = base + kDecTile > len || base < 0;
     if (wl >= 0) need_mask = need_mask || !((base + kDecTile - 1 < wg) || (base >= len - wl));
     auto allowed = [&](int key_in_tile) -> bool {
       const int key = base + key_in_tile;
-      bool ok = key < len;
+      bool ok = key < len && base >= 0;
       if (wl >= 0) ok = ok && (key < wg || key >= len - wl);
       return ok;
     };
@@ -156,7 +167,7 @@ decode_merge_kernel(const DecodeParams p, int D) {
   if (p.block_idx) {
     const int kvh = h / (p.hq / p.hkv);
     const int cnt = p.block_cnt ? min(p.block_cnt[b * p.hkv + kvh], p.max_blocks) : p.max_blocks;
-    nvalid = len > 0 ? (cnt + p.split_blocks - 1) / p.split_blocks : 0;
+    nvalid = len > 0 ? (cnt + p.add_last + p.split_blocks - 1) / p.split_blocks : 0;
   } else {
     nvalid = (len + p.split_tokens - 1) / p.split_tokens;
   }

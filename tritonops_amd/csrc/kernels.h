@@ -49,6 +49,7 @@ struct DecodeParams {
   int64_t bi_sb, bi_sh;
   int32_t max_blocks, split_blocks;
   int32_t win_local, win_global;
+  int32_t add_last;  // implicit extra entry: the block of token len-1
 };
 
 // dtype: 0 bf16, 1 f16.  head_dim in {64, 96, 128}.  Return hipError_t as int.

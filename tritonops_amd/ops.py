@@ -233,7 +233,7 @@ def flash_attn_sparse_triton(q, k, v, cu_seqlens, softmax_scale=None, local_wind
 
 def _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, return_lse,
             block_idx=None, block_cnt=None, bi_strides=(0, 0), max_blocks=0, split_blocks=0,
-            window=(-1, -1)):
+            window=(-1, -1), include_last=False):
     _require_gpu(q, k, v, cu_seq_lens, seq_lens)
     lib = _lib.load()
     q, k, v = _inner_contig(q), _inner_contig(k), _inner_contig(v)
@@ -270,6 +270,7 @@ def _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, re
         a.block_idx_stride_b, a.block_idx_stride_h = bi_strides
         a.max_blocks, a.block_size, a.split_blocks = int(max_blocks), _masks.BLOCK, int(split_blocks)
         a.window_local, a.window_global = window
+        a.include_last_block = 1 if include_last else 0
     nbytes = lib.mi_decode_workspace_bytes(C.byref(a))
     if nbytes == 0:
         raise _lib.MiAttnError(lib.mi_decode_validate(C.byref(a)), lib.mi_last_error().decode())
@@ -345,22 +346,13 @@ def flash_attention_sparse_decoding(q, k, v, cu_seq_lens, global_window_size=64,
         return _decode(q, k, v, None, lens, scale, None, None, return_lse, block_idx=idx, block_cnt=cnt,
                        bi_strides=(cap, 0), max_blocks=cap,
                        split_blocks=split_blocks or max(1, min(8, cap)), window=(lw, gw))
-    idx = block_indices.to(torch.int32)
+    idx = block_indices.to(torch.int32).contiguous()
     if idx.dim() != 3 or idx.shape[0] != B or idx.shape[1] != Hkv:
         raise ValueError("block_indices must be [B, Hkv, n]")
     n = idx.shape[2]
-    cnt = block_counts.to(torch.int32) if block_counts is not None else torch.full(
-        (B, Hkv), n, device=q.device, dtype=torch.int32)
-    if include_last_block:
-        last = torch.clamp((lens - 1) // _masks.BLOCK, min=0)[:, None, None].expand(B, Hkv, 1)
-        slot = torch.arange(n, device=q.device)[None, None, :]
-        present = ((idx == last) & (slot < cnt[..., None])).any(-1)
-        idx = torch.cat([idx, last.to(torch.int32)], dim=2)
-        # put the extra entry right after the valid ones
-        idx = idx.scatter(2, cnt[..., None].to(torch.int64), last.to(torch.int32))
-        cnt = cnt + (~present).to(torch.int32)
-        n += 1
-    idx = idx.contiguous()
-    cnt = cnt.contiguous()
+    cnt = block_counts.to(torch.int32).contiguous() if block_counts is not None else None
+    # the block of the newest token is appended (and de-duplicated) by the kernel
+    total = n + (1 if include_last_block else 0)
     return _decode(q, k, v, None, lens, scale, None, None, return_lse, block_idx=idx, block_cnt=cnt,
-                   bi_strides=(Hkv * n, n), max_blocks=n, split_blocks=split_blocks or max(1, min(8, n)))
+                   bi_strides=(Hkv * n, n), max_blocks=n, split_blocks=split_blocks or max(1, min(8, total)),
+                   include_last=bool(include_last_block))
