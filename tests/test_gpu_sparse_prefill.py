@@ -31,7 +31,7 @@ def test_window_sparse_matches_oracle(lw, gw):
     assert (lse.cpu()[fin] - want_lse[fin]).abs().max() <= LSE_TOL
     if lw >= 5000 or gw >= 5000:       # window covers everything -> dense causal
         dense = ta.flash_attention(q.cuda(), k.cuda(), v.cuda(), cu.cuda())
-        assert_close(got, dense, 4e-3)
+        assert_close(got, dense, 1e-2)   # two kernels, two summation orders: one bf16 ulp of |o| < 2
     if (lw, gw) == (1, 0):             # only the diagonal -> o = v
         G = q.shape[2] // v.shape[2]
         assert_close(got, v.repeat_interleave(G, 2), 1e-6)
@@ -87,7 +87,7 @@ def test_full_lower_triangle_equals_dense():
     m = np.tril(np.ones((9, 9), dtype=bool))
     got, lse = ta.flash_attn_sparse_triton(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), block_mask=m)
     dense, dlse = ta.flash_attn_triton_fwd(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), 64 ** -0.5 * ta.LOG2E)
-    assert_close(got, dense, 4e-3)
+    assert_close(got, dense, 1e-2)   # one bf16 ulp of |o| < 2
     assert (lse - dlse).abs().max().item() <= LSE_TOL
 
 

@@ -64,5 +64,8 @@ constexpr int kSparseRows = 64;
 // LDS stages (KV tiles resident per workgroup) of the two prefill kernels.
 constexpr int kDenseStages = 3;
 constexpr int kSparseStages = 2;
+// Keys per LDS tile of the block-sparse kernel: a 64-key block is walked as two
+// 32-key tiles so that four 2-wave workgroups (8 waves) fit one CU's LDS.
+constexpr int kSparseTileKeys = 32;
 
 }  // namespace mi

@@ -32,17 +32,18 @@ using ic = std::integral_constant<int, V>;
 // vmcnt(N) expcnt(7) lgkmcnt(15) for s_waitcnt on gfx9-family encodings
 constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
 
-// NW wavefronts per workgroup, NS LDS stages (tiles in flight + the one in use).
-template <typename T, int D, int NW, int NS, bool SPARSE>
+// NW wavefronts per workgroup, NS LDS stages (tiles in flight + the one in
+// use), TN keys per tile (64, or 32 so that more workgroups fit one CU's LDS).
+template <typename T, int D, int NW, int NS, int TN, bool SPARSE>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2)))
 prefill_kernel(const PrefillParams p) {
   using G = RowGeom<D>;
   using F = SwizzledFrags<D>;
   constexpr int BM = 32 * NW;
-  constexpr int TILEB = kTileN * F::ROWB;   // one K or V tile
+  constexpr int TILEB = TN * F::ROWB;   // one K or V tile
   constexpr int VBASE = NS * TILEB;         // LDS: NS K tiles, then NS V tiles
   constexpr int RPI = 1024 / F::ROWB;       // tile rows filled by one direct-to-LDS instruction
-  constexpr int NINST = kTileN / RPI;       // such instructions per tensor per tile
+  constexpr int NINST = TN / RPI;       // such instructions per tensor per tile
   constexpr int IPW = NINST / NW;           // ... per wavefront
   static_assert(NINST % NW == 0, "tile rows must split evenly over the waves");
   constexpr int OROWB = D * 2 + 16;         // epilogue staging row
@@ -114,11 +115,12 @@ prefill_kernel(const PrefillParams p) {
   if constexpr (SPARSE) {
     const int32_t* rp = p.row_ptr + b * p.rp_sb + h * p.rp_sh;
     const int beg = rp[qt];
-    n_tiles = rp[qt + 1] - beg;
+    n_tiles = (rp[qt + 1] - beg) * (kTileN / TN);  // a 64-key block is TN-key tiles
     cols = p.col_idx + b * p.ci_sb + h * p.ci_sh + beg;
   } else {
-    n_tiles = (len + kTileN - 1) / kTileN;
-    if (p.causal) n_tiles = min(n_tiles, (q0 + BM + kTileN - 1) / kTileN);
+    static_assert(SPARSE || TN == kTileN, "dense kernel walks 64-key tiles");
+    n_tiles = (len + TN - 1) / TN;
+    if (p.causal) n_tiles = min(n_tiles, (q0 + BM + TN - 1) / TN);
   }
 
   // ---- Q^T operands: lane (query lq, half lh) holds d = 16c + 8lh .. +7
@@ -140,14 +142,19 @@ prefill_kernel(const PrefillParams p) {
   // SLOTS, which must receive logical chunk dslot ^ swz(row) of that row.
   const int drow = lane / F::SLOTS, dslot = lane % F::SLOTS;
   const int64_t k_rowb = p.k_ss * 2, v_rowb = p.v_ss * 2;  // bytes between keys
-  auto dma_tile = [&](int col, auto stage_c) {
+  // first key of tile `it` of this workgroup's list
+  auto tile_k0 = [&](int it) -> int {
+    if (!SPARSE) return it * TN;
+    constexpr int PER = kTileN / TN;
+    return cols[it / PER] * kTileN + (it % PER) * TN;
+  };
+  auto dma_tile = [&](int k0, auto stage_c) {
     constexpr int ST = decltype(stage_c)::value;
-    const int k0 = col * kTileN;
     const char* kt = reinterpret_cast<const char*>(kp) + k0 * k_rowb;
     const char* vt = reinterpret_cast<const char*>(vp) + k0 * v_rowb;
     unsigned char* sK = smem + ST * TILEB;
     unsigned char* sV = smem + VBASE + ST * TILEB;
-    if (k0 + kTileN <= len) {
+    if (k0 + TN <= len) {
       // whole tile inside the sequence: uniform base + 32-bit lane offset
 #pragma unroll
       for (int t = 0; t < IPW; ++t) {
@@ -183,18 +190,17 @@ prefill_kernel(const PrefillParams p) {
 
   auto step = [&](auto stage_c, int it) {
     constexpr int ST = decltype(stage_c)::value;
-    const int col = SPARSE ? cols[it] : it;
     // refill the stage that was read in the previous iteration
     const bool refill = it + NS - 1 < n_tiles;
-    if (refill) dma_tile(SPARSE ? cols[it + NS - 1] : it + NS - 1, ic<(ST + NS - 1) % NS>{});
+    if (refill) dma_tile(tile_k0(it + NS - 1), ic<(ST + NS - 1) % NS>{});
 
-    const int k0 = col * kTileN;
+    const int k0 = tile_k0(it);
     // whole tile above the diagonal for this wave: nothing to add
     const bool skip = p.causal && k0 > q0w + 31;
     if (!skip) {
-      bool need_mask = (k0 + kTileN > len) || (p.causal && k0 + kTileN - 1 > q0w);
+      bool need_mask = (k0 + TN > len) || (p.causal && k0 + TN - 1 > q0w);
       const int wl = p.win_local, wg = p.win_global;
-      if (SPARSE && wl >= 0) need_mask = need_mask || !((k0 + kTileN - 1 < wg) || (q0w + 31 - k0 < wl));
+      if (SPARSE && wl >= 0) need_mask = need_mask || !((k0 + TN - 1 < wg) || (q0w + 31 - k0 < wl));
       const int causal = p.causal;
       auto allowed = [&](int key_in_tile) -> bool {
         const int key = k0 + key_in_tile;
@@ -203,7 +209,7 @@ prefill_kernel(const PrefillParams p) {
         return ok;
       };
       // V addresses carry VBASE inside the lane offsets (see fr.init)
-      compute_tile<T, D, 2>(smem + ST * TILEB, smem + ST * TILEB, fr, Qf, O, m, l, p.scale, need_mask, allowed);
+      compute_tile<T, D, TN / 32>(smem + ST * TILEB, smem + ST * TILEB, fr, Qf, O, m, l, p.scale, need_mask, allowed);
     }
     // The next tile must have landed and everyone must be done with this one.
     // This wave's loads complete in order, so it is enough that at most the
@@ -218,9 +224,9 @@ prefill_kernel(const PrefillParams p) {
 #pragma unroll
   for (int s0 = 0; s0 < NS - 1; ++s0)
     if (s0 < n_tiles) {
-      if (s0 == 0) dma_tile(SPARSE ? cols[0] : 0, ic<0>{});
-      if (s0 == 1) dma_tile(SPARSE ? cols[1] : 1, ic<1 % NS>{});
-      if (s0 == 2) dma_tile(SPARSE ? cols[2] : 2, ic<2 % NS>{});
+      if (s0 == 0) dma_tile(tile_k0(0), ic<0>{});
+      if (s0 == 1) dma_tile(tile_k0(1), ic<1 % NS>{});
+      if (s0 == 2) dma_tile(tile_k0(2), ic<2 % NS>{});
     }
   // tile 0 (and the Q loads issued before it) must be complete
   if (n_tiles >= NS - 1)
@@ -270,9 +276,9 @@ prefill_kernel(const PrefillParams p) {
   }
 }
 
-template <int D, int NW, int NS>
+template <int D, int NW, int NS, int TN>
 constexpr size_t prefill_lds_bytes() {
-  const size_t pipe = (size_t)NS * 2 * kTileN * SwizzledFrags<D>::ROWB;
+  const size_t pipe = (size_t)NS * 2 * TN * SwizzledFrags<D>::ROWB;
   const size_t epi = (size_t)NW * 32 * (D * 2 + 16);
   return pipe > epi ? pipe : epi;
 }
@@ -280,8 +286,9 @@ constexpr size_t prefill_lds_bytes() {
 template <typename T, int D, int NW, bool SPARSE>
 int launch_one(const PrefillParams& p, hipStream_t s) {
   constexpr int NS = SPARSE ? kSparseStages : kDenseStages;
-  auto kern = prefill_kernel<T, D, NW, NS, SPARSE>;
-  constexpr size_t lds = prefill_lds_bytes<D, NW, NS>();
+  constexpr int TN = SPARSE ? kSparseTileKeys : kTileN;
+  auto kern = prefill_kernel<T, D, NW, NS, TN, SPARSE>;
+  constexpr size_t lds = prefill_lds_bytes<D, NW, NS, TN>();
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return (int)e;
