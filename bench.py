@@ -174,14 +174,36 @@ def run_block_sparse(steps, warmup):
     q, k, v = (_randn((B, H, S, D), s) for s in (0, 1, 2))
     fn = lambda: ta.flash_attn_sparse_triton(q, k, v, None, row_ptr=row_ptr, col_idx=col_idx, csr_strides=strides)
     ms = _time_steps(fn, steps, warmup)
+    from tritonops_amd import _lib
+    o = torch.empty_like(q)
+    lse = torch.empty((B, H, S), device="cuda", dtype=torch.float32)
+    a = _lib.AttnSparseArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _lib.MI_DTYPE_BF16
+    a.q, a.k, a.v, a.o, a.lse = (t.data_ptr() for t in (q, k, v, o, lse))
+    for n, t in (("q", q), ("k", k), ("v", v), ("o", o)):
+        setattr(a, n + "_stride_b", t.stride(0))
+        setattr(a, n + "_stride_h", t.stride(1))
+        setattr(a, n + "_stride_s", t.stride(2))
+    a.lse_stride_b, a.lse_stride_h, a.lse_stride_s = lse.stride(0), lse.stride(1), lse.stride(2)
+    a.cu_seqlens = None
+    a.row_ptr, a.col_idx = row_ptr.data_ptr(), col_idx.data_ptr()
+    a.row_ptr_stride_b, a.row_ptr_stride_h, a.col_idx_stride_b, a.col_idx_stride_h = strides
+    a.batch, a.heads_q, a.heads_kv, a.max_seqlen, a.head_dim = B, H, H, S, D
+    a.block_size, a.window_local, a.window_global = 64, -1, -1
+    a.scale_log2 = D ** -0.5 * 1.4426950408889634
+    kms = _event_ms(1, a, steps, warmup)
     flop = 4.0 * D * ((live - nb) * 64 * 64 + nb * 64 * 65 / 2) * B * H
     return {
-        "name": "block_sparse", "ms_per_step": ms, "kernel_ms": ms,
+        "name": "block_sparse", "ms_per_step": ms, "kernel_ms": kms,
         "metric": "sparse_attn_fwd_tflops", "unit": "TFLOP/s", "value": flop / (ms * 1e-3) / 1e12,
-        "roofline": {"bound": "mfma", "achieved": flop / (ms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
+        "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "kernel": "prefill_kernel<bf16,128,sparse>"},
         "config": {"workload": "block-sparse causal fwd bf16 B=2 H=16 S=16384 D=128, 64x64 blocks, band 8 + 4 sink + 10%% (%d live blocks)" % live,
-                   "flop_per_step": flop},
+                   "flop_per_step": flop,
+                   "kv_tile_bytes_per_step": float(live * 64 * D * 2 * 2 * B * H),
+                   "note": "every live 64x64 block re-reads its 32 KiB of K/V from L2 / last-level cache: 64 FLOP per "
+                           "byte moved, so this workload is bound by cache bandwidth well before the MFMA peak"},
     }
 
 
@@ -198,14 +220,39 @@ def run_sparse_decode(steps, warmup):
     fn = lambda: ta.flash_attention_sparse_decoding(q, kc.transpose(1, 2), vc.transpose(1, 2), None,
                                                     seq_lens=lens_d, block_indices=idx)
     ms = _time_steps(fn, steps, warmup)
+    from tritonops_amd import _lib
+    lib = _lib.load()
+    k, v = kc.transpose(1, 2), vc.transpose(1, 2)
+    o = torch.empty((B, Hq, D), device="cuda", dtype=torch.bfloat16)
+    a = _lib.DecodeArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _lib.MI_DTYPE_BF16
+    a.q, a.k, a.v, a.o, a.lse = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), None
+    a.q_stride_b, a.q_stride_h = q.stride(0), q.stride(1)
+    a.k_stride_b, a.k_stride_s, a.k_stride_h = k.stride(0), k.stride(1), k.stride(2)
+    a.v_stride_b, a.v_stride_s, a.v_stride_h = v.stride(0), v.stride(1), v.stride(2)
+    a.o_stride_b, a.o_stride_h = o.stride(0), o.stride(1)
+    a.seq_lens, a.cu_seqlens = lens_d.data_ptr(), None
+    a.batch, a.heads_q, a.heads_kv, a.max_seqlen, a.head_dim = B, Hq, Hkv, L, D
+    a.scale_log2 = D ** -0.5 * 1.4426950408889634
+    a.split_tokens = 64
+    a.block_idx, a.block_cnt = idx.data_ptr(), None
+    a.block_idx_stride_b, a.block_idx_stride_h = Hkv * 128, 128
+    a.max_blocks, a.block_size, a.split_blocks = 128, 64, 8
+    a.window_local = a.window_global = -1
+    a.include_last_block = 1
+    nb = lib.mi_decode_workspace_bytes(C.byref(a))
+    ws = torch.empty(nb, device="cuda", dtype=torch.uint8)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), nb
+    kms = _event_ms(3, a, steps, warmup)
     nbytes_alg = float(B * Hkv * 129 * 64 * D * 2 * 2)
     return {
-        "name": "sparse_decode", "ms_per_step": ms, "kernel_ms": ms,
+        "name": "sparse_decode", "ms_per_step": ms, "kernel_ms": kms,
         "metric": "sparse_decode_hbm_gbs", "unit": "GB/s", "value": nbytes_alg / (ms * 1e-3) / 1e9,
-        "roofline": {"bound": "hbm", "achieved": nbytes_alg / (ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+        "roofline": {"bound": "hbm", "achieved": nbytes_alg / (kms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "kernel": "decode_splitkv_kernel<bf16,128> (block list)"},
         "config": {"workload": "block-sparse decode bf16 B=32 Hq=32 Hkv=8 KV=131072 D=128, top-128 of 64-token blocks + last block",
-                   "bytes_per_step": nbytes_alg, "note": "kernel_ms here is wall time of both passes plus the index preparation"},
+                   "bytes_per_step": nbytes_alg},
     }
 
 
@@ -235,23 +282,23 @@ def cpu_baseline(name):
         return sorted(ts)[len(ts) // 2]
 
     if name == "dense_causal":
-        B, H, S, D = 1, 2, 4096, 128
+        B, H, S, D = 1, 16, 8192, 128
         q, k, v = (torch.randn((B, H, S, D), generator=g).to(torch.bfloat16) for _ in range(3))
         t = med(lambda: orc.causal_attention(q, k, v))
         flop = 2.0 * B * H * S * (S + 1) * D
         return {"value": flop / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
-                "sample": "torch-CPU bf16 causal softmax(qk^T/sqrt(d))v (tutorial/4.4 oracle) on B=1 H=2 S=4096 D=128, "
+                "sample": "torch-CPU bf16 causal softmax(qk^T/sqrt(d))v (tutorial/4.4 oracle) on B=1 H=16 S=8192 D=128 (1/8 of the workload), "
                           "median of 3; same algorithmic-FLOP formula as the GPU figure",
                 "seconds": t}
     if name == "gqa_decode":
-        B, Hq, Hkv, L, D = 2, 32, 8, 32768, 128
+        B, Hq, Hkv, L, D = 8, 32, 8, 32768, 128
         lens = torch.randint(16384, L + 1, (B,), generator=g, dtype=torch.int32)
         q = torch.randn((B, Hq, D), generator=g).to(torch.bfloat16)
         k, v = (torch.randn((B, L, Hkv, D), generator=g).to(torch.bfloat16) for _ in range(2))
         t = med(lambda: orc.flash_attn_decoding_torch(q, k, v, lens))
         nb = float(lens.sum()) * Hkv * 2 * D * 2
         return {"value": nb / t / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
-                "sample": "torch-CPU bf16 decode oracle (flash_attn_decoding.py:339-368) on B=2 of the same shape, median of 3",
+                "sample": "torch-CPU bf16 decode oracle (flash_attn_decoding.py:339-368) on B=8 of the 64 sequences, median of 3",
                 "seconds": t}
     return None
 
@@ -259,10 +306,13 @@ def cpu_baseline(name):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all", choices=["all"] + list(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also launch one elementwise copy of 1 GiB (2 GiB of HBM traffic) as the reference "
+                         "dispatch for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the attention path shards over batch and "
@@ -272,13 +322,23 @@ def main():
     from tritonops_amd import _lib
     _lib.load()   # fail loudly when the HIP library is missing
 
+    if a.traffic_probe:
+        src = torch.ones(1 << 29, device="cuda", dtype=torch.bfloat16)
+        dst = torch.empty_like(src)
+        torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
+    traffic = {}
+    tfile = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tfile):
+        traffic = json.load(open(tfile))   # bytes per launch measured with rocprofv3 --pmc (see profiles/)
     names = list(WORKLOADS) if a.workload == "all" else [a.workload]
     results = []
     for n in names:
         r = WORKLOADS[n](a.steps, a.warmup)
         rf = r["roofline"]
         rf["frac"] = rf["achieved"] / rf["peak"]
-        rf["traffic"] = None
+        rf["traffic"] = traffic.get(r["name"], {}).get("hbm_bytes_per_launch")
         results.append(r)
         torch.cuda.empty_cache()
     head = results[0]
