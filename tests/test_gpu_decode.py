@@ -137,3 +137,26 @@ def test_full_size_decode_properties():
     vc.fill_(0.5)
     got = ta.flash_attention_decoding(q, kc.transpose(1, 2), vc.transpose(1, 2), None, seq_lens=lens.cuda())
     assert (got.float() - 0.5).abs().max().item() <= 4e-3
+
+
+def test_last_block_listed_and_implicit_counts_once():
+    """include_last_block with the last block already in the list (and a ragged
+    count) must equal the oracle, which attends each token at most once."""
+    import tritonops_amd as ta
+
+    B, Hq, Hkv, D, L = 2, 8, 2, 64, 1000
+    lens = torch.tensor([1000, 515], dtype=torch.int32)      # last blocks 15 and 8 (partial)
+    q = randn((B, Hq, D), 1)
+    k, v = _kv(B, L, Hkv, D, torch.bfloat16, 2)
+    idx = torch.tensor([[[3, 15, 0], [15, 0, 0]], [[8, 2, 0], [1, 8, 4]]], dtype=torch.int32)
+    cnt = torch.tensor([[2, 1], [2, 3]], dtype=torch.int32)
+    want = orc.block_sparse_decoding(q, k, v, lens, idx, cnt, include_last_block=True, faithful=False)
+    for sb in (1, 2, 8):
+        got = ta.flash_attention_sparse_decoding(q.cuda(), k.cuda(), v.cuda(), None, seq_lens=lens.cuda(),
+                                                 block_indices=idx.cuda(), block_counts=cnt.cuda(), split_blocks=sb)
+        assert_close(got, want, TOL, "split_blocks=%d" % sb)
+    no_last = orc.block_sparse_decoding(q, k, v, lens, idx, cnt, include_last_block=False, faithful=False)
+    got = ta.flash_attention_sparse_decoding(q.cuda(), k.cuda(), v.cuda(), None, seq_lens=lens.cuda(),
+                                             block_indices=idx.cuda(), block_counts=cnt.cuda(),
+                                             include_last_block=False)
+    assert_close(got, no_last, TOL)

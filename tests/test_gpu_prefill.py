@@ -165,3 +165,22 @@ def test_full_size_properties():
     ref = torch.einsum("bhij,bhjd->bhid", torch.softmax(s, -1), v.float())
     assert_close(o[:, :, rows], ref, TOL)
     assert (lse[:, :, rows] - torch.logsumexp(s, -1) * orc.LOG2E).abs().max().item() <= LSE_TOL
+
+
+def test_long_ragged_batch_with_many_tiles():
+    """Several hundred KV tiles per sequence, lengths straddling every tile and
+    workgroup edge (63/64/65, 255/256/257 ...), packed layout, GQA 4."""
+    import tritonops_amd as ta
+
+    lens = torch.tensor([63, 64, 65, 255, 256, 257, 1023, 1025, 2048, 3000], dtype=torch.int32)
+    cu = cu_from(lens)
+    T = int(cu[-1])
+    q, k, v = randn((1, T, 8, 128), 1), randn((1, T, 2, 128), 2), randn((1, T, 2, 128), 3)
+    want, want_lse = orc.flash_attn_torch(q, k, v, cu, faithful=False, return_lse=True)
+    got, lse = ta.flash_attn_triton_fwd(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), 128 ** -0.5 * ta.LOG2E,
+                                        max_seq_len=3000)
+    assert_close(got, want, TOL)
+    _lse_close(lse, want_lse)
+    nc = ta.flash_attention(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), causal=False)
+    want_nc = orc.varlen_masked_attention(q, k, v, cu, lambda L: torch.ones(L, L, dtype=torch.bool), faithful=False)
+    assert_close(nc, want_nc, TOL)

@@ -115,3 +115,19 @@ def test_batched_layout_full_size_mask():
         ref = torch.einsum("bhij,bhjd->bhid", torch.softmax(s, -1), v.float())
         assert_close(o[:, :, rows], ref, TOL)
         assert (lse[:, :, rows] - torch.logsumexp(s, -1) * orc.LOG2E).abs().max().item() <= LSE_TOL
+
+
+@pytest.mark.parametrize("D,dtype", [(64, torch.float16), (128, torch.float16), (64, torch.bfloat16)])
+def test_sparse_other_dtypes_and_head_dims(D, dtype):
+    import tritonops_amd as ta
+    from tritonops_amd import masks
+
+    q, k, v, cu = _inputs(3, 400, 6, 3, D, dtype)
+    want = orc.flash_attn_sparse_torch(q, k, v, cu, None, 96, 64, faithful=False)
+    got, _ = ta.flash_attn_sparse_triton(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), None, 96, 64)
+    assert got.dtype == dtype
+    assert_close(got, want, TOL)
+    m = masks.synthetic_block_mask(7, band=2, sink=1, frac=0.3, seed=4)
+    want = orc.block_sparse_attention(q, k, v, cu, m, faithful=False)
+    got, _ = ta.flash_attn_sparse_triton(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), block_mask=m)
+    assert_close(got, want, TOL)
