@@ -51,6 +51,10 @@ int check_prefill_strides(const A* a) {
                        a->v_stride_s, a->v_stride_h, a->o_stride_s, a->o_stride_h};
   for (int64_t x : s)
     if (!mult8(x)) return fail(MI_ERR_STRIDE, "q/k/v/o strides must be multiples of 8 elements (got %lld)", (long long)x);
+  // the tile loads address a 64-key tile as scalar base + 32-bit lane offset
+  if (a->k_stride_s < 0 || a->v_stride_s < 0 || a->k_stride_s >= (1 << 24) || a->v_stride_s >= (1 << 24))
+    return fail(MI_ERR_STRIDE, "k/v sequence strides must be in [0, 2^24) elements (got %lld, %lld)",
+                (long long)a->k_stride_s, (long long)a->v_stride_s);
   if (!a->cu_seqlens) {
     const int64_t sb[] = {a->q_stride_b, a->k_stride_b, a->v_stride_b, a->o_stride_b};
     for (int64_t x : sb)

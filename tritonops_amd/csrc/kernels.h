@@ -22,6 +22,7 @@ struct PrefillParams {
   int64_t rp_sb, rp_sh, ci_sb, ci_sh;
   int32_t batch, hq, hkv, max_seqlen;
   int32_t n_qtiles;  // ceil(max_seqlen / rows per workgroup)
+  int32_t n_items;   // logical workgroups = n_qtiles * hq * batch (set by the launcher)
   int32_t causal;
   int32_t win_local, win_global;  // -1 => off
   float scale;                    // log2 domain
@@ -62,7 +63,7 @@ int launch_decode_merge(const DecodeParams& p, int dtype, int head_dim, hipStrea
 constexpr int kDenseRows = 256;
 constexpr int kSparseRows = 64;
 // LDS stages (KV tiles resident per workgroup) of the two prefill kernels.
-constexpr int kDenseStages = 3;
+constexpr int kDenseStages = 4;
 constexpr int kSparseStages = 2;
 // Keys per LDS tile of the block-sparse kernel: a 64-key block is walked as two
 // 32-key tiles so that four 2-wave workgroups (8 waves) fit one CU's LDS.

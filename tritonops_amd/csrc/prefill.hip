@@ -34,9 +34,11 @@ constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (7 << 4)
 
 // NW wavefronts per workgroup, NS LDS stages (tiles in flight + the one in
 // use), TN keys per tile (64, or 32 so that more workgroups fit one CU's LDS).
+extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+// One work item: the q tile that logical workgroup id `bid` stands for.
 template <typename T, int D, int NW, int NS, int TN, bool SPARSE>
-__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2)))
-prefill_kernel(const PrefillParams p) {
+__device__ __forceinline__ void prefill_item(const PrefillParams p, const int bid) {
   using G = RowGeom<D>;
   using F = SwizzledFrags<D>;
   constexpr int BM = 32 * NW;
@@ -47,8 +49,6 @@ prefill_kernel(const PrefillParams p) {
   constexpr int IPW = NINST / NW;           // ... per wavefront
   static_assert(NINST % NW == 0, "tile rows must split evenly over the waves");
   constexpr int OROWB = D * 2 + 16;         // epilogue staging row
-
-  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -63,7 +63,6 @@ prefill_kernel(const PrefillParams p) {
   const int n_units = p.batch * p.hkv;
   int unit, s;
   {
-    const int bid = blockIdx.x;
     if ((n_units & 7) == 0) {
       const int xcd = bid & 7, slot = bid >> 3;
       unit = (slot / per_unit) * 8 + xcd;
@@ -105,7 +104,7 @@ prefill_kernel(const PrefillParams p) {
   T* op = reinterpret_cast<T*>(p.o) + o_off + h * p.o_sh;
 
   F fr;
-  fr.init(lane, VBASE);
+  fr.init(lane, (uint32_t)(uintptr_t)smem, VBASE);
   const int q0w = q0 + 32 * wave;
   const int qrow = q0w + fr.lq;
 
@@ -143,32 +142,63 @@ prefill_kernel(const PrefillParams p) {
   const int drow = lane / F::SLOTS, dslot = lane % F::SLOTS;
   const int64_t k_rowb = p.k_ss * 2, v_rowb = p.v_ss * 2;  // bytes between keys
   // first key of tile `it` of this workgroup's list
-  auto tile_k0 = [&](int it) -> int {
+  auto tile_k0 = [&](int it) __attribute__((always_inline)) -> int {
     if (!SPARSE) return it * TN;
     constexpr int PER = kTileN / TN;
     return cols[it / PER] * kTileN + (it % PER) * TN;
   };
-  auto dma_tile = [&](int k0, auto stage_c) {
+  // The load is issued from inline assembly on purpose: the compiler then does
+  // not know that LDS writes are in flight.  When it knows, it makes every
+  // transposing LDS read wait for ALL outstanding loads (vmcnt(0)), the tile
+  // requested a moment ago included, which turns the multi-stage pipeline into
+  // a synchronous copy.  Completion is tracked by hand instead: this wave's
+  // loads retire in order, so "at most n younger loads outstanding" (the
+  // counted vmcnt waits below) followed by the workgroup barrier publishes a
+  // tile.  M0 carries the LDS byte address of the 1 KiB slab.
+  const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem);
+  auto dma16 = [&](const char* g, uint32_t slab) __attribute__((always_inline)) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(g), "s"(slab)
+                 : "memory");
+  };
+  // A tile load address is (uniform tensor base + uniform tile offset), both
+  // kept in scalar registers, plus a per-lane 32-bit offset that is fixed for
+  // the whole item: two vector instructions per load instead of a 64-bit
+  // multiply-add chain.
+  auto uniform64 = [](uint64_t x) __attribute__((always_inline)) -> uint64_t {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)x);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(x >> 32));
+    return ((uint64_t)hi << 32) | lo;
+  };
+  const uint32_t k_pitch = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)k_rowb);
+  const uint32_t v_pitch = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)v_rowb);
+  const uint64_t k_base = uniform64((uint64_t)(uintptr_t)kp);
+  const uint64_t v_base = uniform64((uint64_t)(uintptr_t)vp);
+  uint32_t koff[IPW], voff[IPW];
+#pragma unroll
+  for (int t = 0; t < IPW; ++t) {
+    const int r = RPI * (wave + NW * t) + drow;
+    koff[t] = (uint32_t)r * k_pitch + (uint32_t)(dslot ^ F::swz_k(r)) * 16u;
+    voff[t] = (uint32_t)r * v_pitch + (uint32_t)(dslot ^ F::swz_v(r)) * 16u;
+  }
+  auto dma_tile = [&](int k0, auto stage_c) __attribute__((always_inline)) {
     constexpr int ST = decltype(stage_c)::value;
     const char* kt = reinterpret_cast<const char*>(kp) + k0 * k_rowb;
     const char* vt = reinterpret_cast<const char*>(vp) + k0 * v_rowb;
-    unsigned char* sK = smem + ST * TILEB;
-    unsigned char* sV = smem + VBASE + ST * TILEB;
+    const uint32_t sK = lds0 + ST * TILEB;
+    const uint32_t sV = lds0 + VBASE + ST * TILEB;
     if (k0 + TN <= len) {
-      // whole tile inside the sequence: uniform base + 32-bit lane offset
+      // whole tile inside the sequence
+      const uint32_t k0u = (uint32_t)__builtin_amdgcn_readfirstlane(k0);
+      const uint64_t kt_u = k_base + (uint64_t)k0u * k_pitch, vt_u = v_base + (uint64_t)k0u * v_pitch;
 #pragma unroll
       for (int t = 0; t < IPW; ++t) {
         const int inst = wave + NW * t;
         const int r = RPI * inst + drow;
         const int kc = dslot ^ F::swz_k(r), vc = dslot ^ F::swz_v(r);
-        const uint32_t kl = (uint32_t)drow * (uint32_t)k_rowb + (uint32_t)kc * 16u;
-        const uint32_t vl = (uint32_t)drow * (uint32_t)v_rowb + (uint32_t)vc * 16u;
-        if (D != 96 || kc < G::NCH)
-          __builtin_amdgcn_global_load_lds((glb_void*)(kt + (RPI * inst) * k_rowb + kl),
-                                           (lds_void*)(sK + inst * 1024), 16, 0, 0);
-        if (D != 96 || vc < G::NCH)
-          __builtin_amdgcn_global_load_lds((glb_void*)(vt + (RPI * inst) * v_rowb + vl),
-                                           (lds_void*)(sV + inst * 1024), 16, 0, 0);
+        if (D != 96 || kc < G::NCH) dma16(reinterpret_cast<const char*>(kt_u + koff[t]), sK + inst * 1024);
+        if (D != 96 || vc < G::NCH) dma16(reinterpret_cast<const char*>(vt_u + voff[t]), sV + inst * 1024);
       }
     } else {
       // rows past the sequence end re-read its last row (masked later)
@@ -179,15 +209,199 @@ prefill_kernel(const PrefillParams p) {
         const int kc = dslot ^ F::swz_k(r), vc = dslot ^ F::swz_v(r);
         const int64_t rr = min(k0 + r, len - 1) - k0;
         if (D != 96 || kc < G::NCH)
-          __builtin_amdgcn_global_load_lds((glb_void*)(kt + rr * k_rowb + kc * 16), (lds_void*)(sK + inst * 1024),
-                                           16, 0, 0);
+          dma16(kt + rr * k_rowb + kc * 16, sK + inst * 1024);
         if (D != 96 || vc < G::NCH)
-          __builtin_amdgcn_global_load_lds((glb_void*)(vt + rr * v_rowb + vc * 16), (lds_void*)(sV + inst * 1024),
-                                           16, 0, 0);
+          dma16(vt + rr * v_rowb + vc * 16, sV + inst * 1024);
       }
     }
   };
 
+  if constexpr (!SPARSE) {
+    // ---- dense: software pipeline over HALF tiles (32 keys) inside each wave.
+    // A stalled MFMA blocks the vector ALU of its SIMD for every wave, so MFMA
+    // and softmax arithmetic only overlap when one wave's instruction stream
+    // interleaves them.  At position h the wave therefore runs, in ONE
+    // straight-line block, the 8 MFMAs of S[h+1] = K Q^T for the next half
+    // together with max / exp2 / convert of the current half S[h]; then
+    // (after the rare deferred rescale of O) the 8 MFMAs of O += V^T P^T for
+    // half h.  K of half h+1 must be in LDS while half h is being finished:
+    // tile t+1 has to be visible before position 2t+1, which the barrier at
+    // the top of tile t guarantees.
+    static_assert(TN == kTileN && NS >= 3, "pipelined dense path: 64-key tiles, >= 3 stages");
+    int H_w = (len + 31) / 32;                        // halves this wave works on
+    if (p.causal) H_w = min(H_w, q0w / 32 + 1);       // nothing above its own diagonal block
+    H_w = min(H_w, 2 * n_tiles);
+    if (q0w >= len) H_w = 0;                          // all rows past the sequence end
+    f32x16 S[2];
+    const int causal = p.causal;
+    const float scale = p.scale;
+    const int row_lim = causal ? min(qrow, len - 1) : len - 1;  // largest key this lane may see
+    constexpr int KR = G::KSTEPS < 4 ? G::KSTEPS : 4;  // K fragments kept in flight
+    i32x4 kf[KR];  // fragments 0..KR-1 of the half that is scored next, read one block ahead
+
+    // keys of half hh that this lane's query must not see -> -inf (rare)
+    auto mask_half = [&](int hh, f32x16& Sx) __attribute__((always_inline)) {
+      const int k0h = hh * 32;
+      if ((k0h + 32 > len) || (causal && k0h + 31 > q0w)) {
+        const int t = row_lim - k0h - 8 * fr.lh;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (16 * (r >> 3) + (r & 7) > t) Sx[r] = -INFINITY;
+      }
+    };
+
+    // The running-max update for the half in Sx, cut into pieces that are
+    // dropped behind successive MFMAs.  After piece 7: m is the reference max
+    // that the exponentials of Sx will use, l is on that scale, and O still
+    // has to be multiplied by alpha when grow is set.
+    float a0, a1, a2, a3, a4, mx, m_new, alpha;
+    bool grow;
+    auto max_piece = [&](int sl, const f32x16& Sx) __attribute__((always_inline)) {
+      if (sl == 1) {
+        a0 = fmaxf(fmaxf(Sx[0], Sx[1]), Sx[2]);
+        a1 = fmaxf(fmaxf(Sx[3], Sx[4]), Sx[5]);
+      } else if (sl == 2) {
+        a2 = fmaxf(fmaxf(Sx[6], Sx[7]), Sx[8]);
+        a3 = fmaxf(fmaxf(Sx[9], Sx[10]), Sx[11]);
+      } else if (sl == 3) {
+        a4 = fmaxf(fmaxf(Sx[12], Sx[13]), Sx[14]);
+        a0 = fmaxf(fmaxf(a0, a1), Sx[15]);
+      } else if (sl == 4) {
+        a2 = fmaxf(fmaxf(a2, a3), a4);
+        mx = fmaxf(a0, a2);
+      } else if (sl == 5) {
+        mx = max_with_other_half(mx);
+      } else if (sl == 6) {
+        m_new = fmaxf(m, mx * scale);
+        grow = __builtin_amdgcn_ballot_w64(m_new > m + kRescaleSlack) != 0;
+      } else if (sl == 7) {
+        const float m_next = grow ? m_new : m;
+        // a lane whose keys were all masked so far keeps m = -inf: factor 0 (l and O are 0)
+        alpha = fast_exp2(m - ((m_next == -INFINITY) ? 0.f : m_next));
+        l *= alpha;
+        m = m_next;
+      }
+    };
+
+    // Position h.  Entry state: S[h&1] holds the scores of half h, m already
+    // includes them and O, l are on the scale of m; kf holds the first K
+    // fragments of half h+1.
+    //   block A: [MFMAs of S(h+1) = K Q^T] interleaved with [exp2 / sum / pack of S(h)]
+    //   block B: [MFMAs of O += V^T P(h)^T] interleaved with [max update for S(h+1)]
+    // sched_barrier(0) after each slice pins the interleaving: one MFMA, the
+    // LDS reads for a slice four positions ahead, and a few VALU instructions.
+    auto half_step = [&](auto j_c, int h) __attribute__((always_inline)) {
+      constexpr int J = decltype(j_c)::value;  // h % (2 NS)
+      if (h >= H_w) return;
+      const bool has_next = h + 1 < H_w;
+      constexpr int TS = J / 2, KB = J & 1;    // stage of tile h/2, which half of it
+      constexpr int KS = KB == 0 ? TS : (TS + 1) % NS;      // stage holding K of half h+1
+      constexpr uint32_t KOFF = KS * TILEB, VOFF = TS * TILEB;
+      constexpr uint32_t K2OFF = ((TS + 1) % NS) * TILEB;   // stage holding K of half h+2
+      f32x16& Sc = S[KB];
+      f32x16& Sn = S[KB ^ 1];
+      const float m_neg = (m == -INFINITY) ? 0.f : -m;
+      uint32_t P[8];
+      i32x4 vf[G::NDB];
+      float rs = 0.f;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        if (c < G::KSTEPS) {
+          const f32x16 acc = (c == 0) ? (f32x16){0} : Sn;
+          Sn = Elem<T>::mfma(kf[c % KR], Qf[c], acc);
+          if (c + KR < G::KSTEPS) kf[c % KR] = fr.load_k(KOFF, KB ^ 1, c + KR);
+        }
+        if (c >= 8 - G::NDB) vf[c - (8 - G::NDB)] = fr.load_v(VOFF, 2 * KB, c - (8 - G::NDB));
+        const float p0 = fast_exp2(fmaf(Sc[2 * c], scale, m_neg));
+        const float p1 = fast_exp2(fmaf(Sc[2 * c + 1], scale, m_neg));
+        rs += p0 + p1;
+        P[c] = Elem<T>::pack2(p0, p1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      l += rs;
+      // keep the exponentials in this block (they would otherwise sink below
+      // the branches that follow, away from the MFMAs they are meant to overlap)
+      asm volatile("" : "+v"(P[0]), "+v"(P[1]), "+v"(P[2]), "+v"(P[3]), "+v"(P[4]), "+v"(P[5]), "+v"(P[6]), "+v"(P[7]), "+v"(l));
+      mask_half(h + 1, Sn);
+      const float m_keep = m, l_keep = l;
+#pragma unroll
+      for (int sl = 0; sl < 8; ++sl) {
+        if (sl < 2 * G::NDB) {
+          const int kk = sl / G::NDB, db = sl % G::NDB;
+          const i32x4 pf = {(int)P[4 * kk], (int)P[4 * kk + 1], (int)P[4 * kk + 2], (int)P[4 * kk + 3]};
+          O[db] = Elem<T>::mfma(vf[db], pf, O[db]);
+          if (kk == 0) vf[db] = fr.load_v(VOFF, 2 * KB + 1, db);
+        }
+        if (sl >= 4 && sl - 4 < KR) kf[sl - 4] = fr.load_k(K2OFF, KB, sl - 4);
+        max_piece(sl, Sn);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // The last half of a wave scored stale LDS contents above (no half h+1
+      // exists); drop that update.
+      m = has_next ? m : m_keep;
+      l = has_next ? l : l_keep;
+      asm volatile("" : "+v"(m), "+v"(l));
+      // rare: the reference max moved, bring O to the new scale
+      if (grow && has_next) {
+#pragma unroll
+        for (int db = 0; db < G::NDB; ++db) O[db] *= alpha;
+      }
+    };
+
+    // tile t: barrier (tile t+1 visible, stage of tile t-1 free), refill, two halves
+    auto tile_iter = [&](auto ts_c, int t) __attribute__((always_inline)) {
+      constexpr int TS = decltype(ts_c)::value;
+      // tile t+1 was requested NS-2 iterations ago; at most NS-3 younger tiles may still fly
+      if (t + NS - 2 < n_tiles)
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 3) * 2 * IPW));
+      else
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+      __syncthreads();
+      if (t + NS - 1 < n_tiles) dma_tile(tile_k0(t + NS - 1), ic<(TS + NS - 1) % NS>{});
+      half_step(ic<2 * TS>{}, 2 * t);
+      half_step(ic<2 * TS + 1>{}, 2 * t + 1);
+    };
+
+#pragma unroll
+    for (int s0 = 0; s0 < NS - 1; ++s0)
+      if (s0 < n_tiles) {
+        if (s0 == 0) dma_tile(tile_k0(0), ic<0>{});
+        if (s0 == 1) dma_tile(tile_k0(1), ic<1 % NS>{});
+        if (s0 == 2) dma_tile(tile_k0(2), ic<2 % NS>{});
+      }
+    // Everything requested so far must have landed: the Q operands and tile 0
+    // are needed now, and an unconditional full wait here also tells the
+    // compiler that no register load is pending inside the loop (it would
+    // otherwise guard the first use of every Q register there with a wait
+    // that also drains the tile loads).
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    __syncthreads();
+    if (H_w > 0) {
+      // scores and running max of half 0, then the first fragments of half 1
+      f32x16 acc = (f32x16){0};
+#pragma unroll
+      for (int c = 0; c < G::KSTEPS; ++c) acc = Elem<T>::mfma(fr.load_k(0u, 0, c), Qf[c], acc);
+      S[0] = acc;
+      mask_half(0, S[0]);
+#pragma unroll
+      for (int sl = 1; sl < 8; ++sl) max_piece(sl, S[0]);
+#pragma unroll
+      for (int c = 0; c < KR; ++c) kf[c] = fr.load_k(0u, 1, c);
+    }
+
+    for (int t = 0; t < n_tiles; t += NS) {
+      tile_iter(ic<0>{}, t);
+      if (t + 1 >= n_tiles) break;
+      tile_iter(ic<1 % NS>{}, t + 1);
+      if (t + 2 >= n_tiles) break;
+      tile_iter(ic<2 % NS>{}, t + 2);
+      if (NS > 3) {
+        if (t + 3 >= n_tiles) break;
+        tile_iter(ic<3 % NS>{}, t + 3);
+      }
+    }
+    __syncthreads();  // the staging below reuses the tile buffers
+  } else {
   auto step = [&](auto stage_c, int it) {
     constexpr int ST = decltype(stage_c)::value;
     // refill the stage that was read in the previous iteration
@@ -209,7 +423,7 @@ prefill_kernel(const PrefillParams p) {
         return ok;
       };
       // V addresses carry VBASE inside the lane offsets (see fr.init)
-      compute_tile<T, D, TN / 32>(smem + ST * TILEB, smem + ST * TILEB, fr, Qf, O, m, l, p.scale, need_mask, allowed);
+      compute_tile<T, D, TN / 32>((uint32_t)(ST * TILEB), (uint32_t)(ST * TILEB), fr, Qf, O, m, l, p.scale, need_mask, allowed);
     }
     // The next tile must have landed and everyone must be done with this one.
     // This wave's loads complete in order, so it is enough that at most the
@@ -245,6 +459,7 @@ prefill_kernel(const PrefillParams p) {
   if (it < n_tiles) step(ic<0>{}, it++);
   if (it < n_tiles) step(ic<1 % NS>{}, it++);
   if (NS > 3 && it < n_tiles) step(ic<2 % NS>{}, it++);
+  }
 
   // ---- epilogue: normalise, transpose through LDS, coalesced 16-byte stores
   const float l_tot = sum_with_other_half(l);
@@ -276,11 +491,47 @@ prefill_kernel(const PrefillParams p) {
   }
 }
 
+// Persistent launch: the grid holds at most as many workgroups as the device
+// runs at once, and each walks the logical workgroup ids id, id + grid, ...
+// Handing a CU its next q tile this way costs a barrier; a fresh workgroup
+// launch left the CU idle for several microseconds (measured ~12 us between
+// the end of one 512-thread, 128 KiB-LDS workgroup and the first instruction
+// of the next).  Odd rounds are walked back to front within each XCD (id & 7
+// is kept): ids run from the longest q tile of a unit to the shortest, so the
+// workgroup that drew a long tile in one round draws a short one in the next,
+// which balances causal work without a shared counter.
+template <typename T, int D, int NW, int NS, int TN, bool SPARSE>
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2)))
+prefill_kernel(const PrefillParams p) {
+  const int grid = gridDim.x;
+  int round = 0;
+  for (int base = 0; base < p.n_items; base += grid, ++round) {
+    int w = blockIdx.x;
+    if ((round & 1) && (grid & 7) == 0) w = (((grid >> 3) - 1 - (w >> 3)) << 3) | (w & 7);
+    const int bid = base + w;
+    if (bid < p.n_items) prefill_item<T, D, NW, NS, TN, SPARSE>(p, bid);
+    if (base + grid < p.n_items) __syncthreads();  // the next item reuses the LDS tiles
+  }
+}
+
 template <int D, int NW, int NS, int TN>
 constexpr size_t prefill_lds_bytes() {
   const size_t pipe = (size_t)NS * 2 * TN * SwizzledFrags<D>::ROWB;
   const size_t epi = (size_t)NW * 32 * (D * 2 + 16);
   return pipe > epi ? pipe : epi;
+}
+
+// CUs of the current device (cached per device; 0 if the query fails)
+inline int device_cu_count() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+    cached[dev] = n > 0 ? n : -1;
+  }
+  return cached[dev] > 0 ? cached[dev] : 0;
 }
 
 template <typename T, int D, int NW, bool SPARSE>
@@ -292,8 +543,16 @@ int launch_one(const PrefillParams& p, hipStream_t s) {
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return (int)e;
-  const long long grid = (long long)p.n_qtiles * p.hq * p.batch;
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, p);
+  PrefillParams pp = p;
+  const long long items = (long long)p.n_qtiles * p.hq * p.batch;
+  pp.n_items = (int)items;
+  long long grid = items;
+  if (!SPARSE) {
+    // one workgroup per CU is resident (LDS); more ids than that are walked in-kernel
+    const int cus = device_cu_count();
+    if (cus > 0 && grid > cus) grid = cus;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, pp);
   return (int)hipGetLastError();
 }
 

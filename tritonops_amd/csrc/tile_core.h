@@ -171,15 +171,24 @@ struct SwizzledFrags {
   uint32_t k_a[G::KSTEPS];  // byte offset of chunk step c inside a 32-key block
   uint32_t v_a[G::NDB][2];  // byte offset of (d block, first/second read) inside a 16-key group
 
-  // v_bias is folded into the V fragment offsets: the V tiles may then live
-  // beyond the 64 KiB reach of a DS immediate while every read still is
-  // "lane register + immediate" relative to the K tile of the same stage.
-  __device__ __forceinline__ void init(int lane, int v_bias) {
+  // The lane registers hold absolute LDS addresses: lds_base is the address of
+  // the first K tile, lds_base + v_bias that of the first V tile (the V tiles
+  // may then live beyond the 64 KiB reach of a DS immediate while every read
+  // still is "lane register + immediate" with the tile offset of its K tile).
+  // Each address is pinned in a register of its own (empty asm): the compiler
+  // would otherwise re-derive them with vector adds inside the loop, or fold
+  // the bias into the immediates and push those past 64 KiB.
+  __device__ __forceinline__ void init(int lane, uint32_t lds_base, int v_bias) {
     lq = lane & 31;
     lh = lane >> 5;
+    v_bias += (int)lds_base;
+    asm volatile("" : "+v"(v_bias));
     const int krow = key_perm(lq);
 #pragma unroll
-    for (int c = 0; c < G::KSTEPS; ++c) k_a[c] = krow * ROWB + (((2 * c + lh) ^ swz_k(krow)) << 4);
+    for (int c = 0; c < G::KSTEPS; ++c) {
+      k_a[c] = lds_base + krow * ROWB + (((2 * c + lh) ^ swz_k(krow)) << 4);
+      asm volatile("" : "+v"(k_a[c]));
+    }
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
       const int r = 8 * lh + 4 * e + ((lane & 15) >> 2);
@@ -187,15 +196,24 @@ struct SwizzledFrags {
       for (int db = 0; db < G::NDB; ++db) {
         const int ch = 4 * db + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
         v_a[db][e] = v_bias + r * ROWB + ((ch ^ swz_v(r)) << 4) + (lane & 1) * 8;
+        asm volatile("" : "+v"(v_a[db][e]));
       }
     }
   }
   // swz_k is invariant under row += 32, swz_v under row += 16
-  __device__ __forceinline__ i32x4 load_k(const unsigned char* sK, int kb, int c) const {
-    return *reinterpret_cast<const i32x4*>(sK + k_a[c] + kb * 32 * ROWB);
+  // tile_off: byte offset of the stage's K tile from the first K tile (the V
+  // tile of the same stage sits at the same offset from the first V tile)
+  __device__ __forceinline__ i32x4 load_k(uint32_t tile_off, int kb, int c) const {
+    typedef __attribute__((address_space(3))) const i32x4 lds_i32x4;
+    return *(lds_i32x4*)(uintptr_t)(k_a[c] + tile_off + kb * 32 * ROWB);
   }
-  __device__ __forceinline__ i32x4 load_v(const unsigned char* sV, int kk, int db) const {
-    return read_tr_pair(sV + v_a[db][0] + kk * 16 * ROWB, sV + v_a[db][1] + kk * 16 * ROWB);
+  __device__ __forceinline__ i32x4 load_v(uint32_t tile_off, int kk, int db) const {
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(uintptr_t)(v_a[db][0] + tile_off + kk * 16 * ROWB));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(uintptr_t)(v_a[db][1] + tile_off + kk * 16 * ROWB));
+    i32x2 l2 = __builtin_bit_cast(i32x2, lo);
+    i32x2 h2 = __builtin_bit_cast(i32x2, hi);
+    i32x4 out = {l2[0], l2[1], h2[0], h2[1]};
+    return out;
   }
 };
 
@@ -208,8 +226,8 @@ constexpr float kRescaleSlack = 8.0f;
 // S^T = K Q^T for a tile of NKB 32-key blocks: NKB independent accumulator
 // chains stepped alternately, K fragments fetched kPrefetch steps ahead of the
 // MFMA that uses them.
-template <typename T, int D, int NKB, typename Frags>
-__device__ __forceinline__ void qk_scores(const unsigned char* sK, const Frags& fr,
+template <typename T, int D, int NKB, typename Frags, typename Tile>
+__device__ __forceinline__ void qk_scores(Tile sK, const Frags& fr,
                                           const i32x4 (&Qf)[RowGeom<D>::KSTEPS], f32x16 (&S)[NKB]) {
   using G = RowGeom<D>;
   constexpr int NSTEP = NKB * G::KSTEPS;
@@ -290,8 +308,8 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&S)[NKB], int lh, f32x16 (&
 }
 
 // O^T += V^T P^T for one tile.
-template <typename T, int D, int NKB, typename Frags>
-__device__ __forceinline__ void pv_accumulate(const unsigned char* sV, const Frags& fr,
+template <typename T, int D, int NKB, typename Frags, typename Tile>
+__device__ __forceinline__ void pv_accumulate(Tile sV, const Frags& fr,
                                               const uint32_t (&P)[NKB][8], f32x16 (&O)[RowGeom<D>::NDB]) {
   using G = RowGeom<D>;
 #pragma unroll
@@ -308,6 +326,7 @@ __device__ __forceinline__ void pv_accumulate(const unsigned char* sV, const Fra
 
 // One KV tile of NKB*32 keys against the wave's 32 queries.
 //   sK, sV : LDS tiles holding the keys of this tile, in the layout of Frags
+//            (pointers for PaddedFrags, byte offsets for SwizzledFrags)
 //   Qf     : B operands of Q^T, chunk c covers d = 16c .. 16c+15
 //   O      : O^T accumulators, block db covers d = 32db .. 32db+31
 //   m      : reference max of the exponent, scaled base-2 domain (-inf at
@@ -315,9 +334,8 @@ __device__ __forceinline__ void pv_accumulate(const unsigned char* sV, const Fra
 //   l      : this lane's share of the running row sum (the other half of the
 //            sum lives in lane l^32; add them at the end)
 //   allowed(key_in_tile) is consulted only when need_mask is true.
-template <typename T, int D, int NKB, typename Frags, typename MaskF>
-__device__ __forceinline__ void compute_tile(const unsigned char* sK, const unsigned char* sV,
-                                             const Frags& fr, const i32x4 (&Qf)[RowGeom<D>::KSTEPS],
+template <typename T, int D, int NKB, typename Frags, typename Tile, typename MaskF>
+__device__ __forceinline__ void compute_tile(Tile sK, Tile sV, const Frags& fr, const i32x4 (&Qf)[RowGeom<D>::KSTEPS],
                                              f32x16 (&O)[RowGeom<D>::NDB], float& m, float& l,
                                              float scale, bool need_mask, MaskF allowed) {
   f32x16 S[NKB];
