@@ -238,7 +238,8 @@ def run_sparse_decode(steps, warmup):
     a.split_tokens = 64
     a.block_idx, a.block_cnt = idx.data_ptr(), None
     a.block_idx_stride_b, a.block_idx_stride_h = Hkv * 128, 128
-    a.max_blocks, a.block_size, a.split_blocks = 128, 64, 8
+    a.max_blocks, a.block_size = 128, 64
+    a.split_blocks = lib.mi_decode_choose_split_blocks(B, Hkv, 129, 256)
     a.window_local = a.window_global = -1
     a.include_last_block = 1
     nb = lib.mi_decode_workspace_bytes(C.byref(a))
@@ -252,7 +253,7 @@ def run_sparse_decode(steps, warmup):
         "roofline": {"bound": "hbm", "achieved": nbytes_alg / (kms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "kernel": "decode_splitkv_kernel<bf16,128> (block list)"},
         "config": {"workload": "block-sparse decode bf16 B=32 Hq=32 Hkv=8 KV=131072 D=128, top-128 of 64-token blocks + last block",
-                   "bytes_per_step": nbytes_alg},
+                   "bytes_per_step": nbytes_alg, "split_blocks": int(a.split_blocks)},
     }
 
 

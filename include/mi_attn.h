@@ -221,6 +221,13 @@ size_t mi_decode_workspace_bytes(const mi_decode_args *args);
  * units for the given problem; host only. */
 int mi_decode_choose_split_tokens(int batch, int heads_kv, int max_seqlen,
                                   int num_cus);
+/* Heuristic chunk length in listed blocks for the block-list form: the largest
+ * number of chunks per (sequence, kv-head) whose wavefronts are all resident
+ * at once on `num_cus` compute units (a second, partly filled round of
+ * wavefronts costs more than longer chunks do); host only.  `total_blocks`
+ * counts the implicit last block when include_last_block is set. */
+int mi_decode_choose_split_blocks(int batch, int heads_kv, int total_blocks,
+                                  int num_cus);
 
 /* Pass 1 only: partials into the workspace. */
 int mi_decode_splitkv(const mi_decode_args *args, void *stream);

@@ -186,6 +186,19 @@ def test_split_heuristic(lib):
     assert f(4096, 8, 4096, 256) == 4096         # plenty of sequences: one chunk each
 
 
+def test_split_blocks_heuristic(lib):
+    f = lib.mi_decode_choose_split_blocks
+    # 32 sequences x 8 kv-heads on 256 CUs: 2048 resident wavefronts / 256 units = 8 chunks of 129 blocks
+    assert f(32, 8, 129, 256) == 17
+    assert f(4096, 8, 129, 256) == 129           # more units than wavefront slots: one chunk each
+    assert f(1, 1, 129, 256) == 1                # one unit: a chunk per block
+    assert f(0, 0, 0, 0) == 1
+    for args in [(32, 8, 129, 256), (3, 5, 77, 256), (64, 8, 2048, 304)]:
+        sb = f(*args)
+        chunks = -(-args[2] // sb)
+        assert 1 <= sb <= args[2] and chunks * args[0] * args[1] <= max(8 * args[3], args[0] * args[1])
+
+
 def test_time_launches_rejects_bad_arguments(lib):
     ms = C.c_float()
     assert lib.mi_time_launches(0, None, None, 0, 1, C.byref(ms)) == -1

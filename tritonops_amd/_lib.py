@@ -98,6 +98,7 @@ EXPORTS = {
     "mi_decode_num_splits": (C.c_int, [C.POINTER(DecodeArgs)]),
     "mi_decode_workspace_bytes": (_sz, [C.POINTER(DecodeArgs)]),
     "mi_decode_choose_split_tokens": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int]),
+    "mi_decode_choose_split_blocks": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int]),
     "mi_decode_splitkv": (C.c_int, [C.POINTER(DecodeArgs), _vp]),
     "mi_decode_merge": (C.c_int, [C.POINTER(DecodeArgs), _vp]),
     "mi_decode": (C.c_int, [C.POINTER(DecodeArgs), _vp]),

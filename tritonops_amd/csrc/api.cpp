@@ -252,6 +252,18 @@ int mi_decode_choose_split_tokens(int batch, int heads_kv, int max_seqlen, int n
   return (int)tokens;
 }
 
+int mi_decode_choose_split_blocks(int batch, int heads_kv, int total_blocks, int num_cus) {
+  // One wavefront per (chunk, kv-head, sequence), 8 wavefronts resident per
+  // compute unit: use as many chunks as fit in one resident round.
+  if (batch <= 0 || heads_kv <= 0 || total_blocks <= 0) return 1;
+  if (num_cus <= 0) num_cus = 256;
+  const long long units = (long long)batch * heads_kv;
+  long long chunks = 8LL * num_cus / units;
+  if (chunks < 1) chunks = 1;
+  if (chunks > total_blocks) chunks = total_blocks;
+  return (int)((total_blocks + chunks - 1) / chunks);
+}
+
 int mi_decode_validate(const mi_decode_args* a) {
   int rc = decode_validate_shape(a);
   if (rc) return rc;

@@ -113,8 +113,9 @@ __device__ __forceinline__ void prefill_item(const PrefillParams p, const int bi
   const int32_t* cols = nullptr;
   if constexpr (SPARSE) {
     const int32_t* rp = p.row_ptr + b * p.rp_sb + h * p.rp_sh;
-    const int beg = rp[qt];
-    n_tiles = (rp[qt + 1] - beg) * (kTileN / TN);  // a 64-key block is TN-key tiles
+    // (values loaded through vector memory: tell the compiler they are uniform)
+    const int beg = __builtin_amdgcn_readfirstlane(rp[qt]);
+    n_tiles = __builtin_amdgcn_readfirstlane(rp[qt + 1] - beg) * (kTileN / TN);  // a 64-key block is TN-key tiles
     cols = p.col_idx + b * p.ci_sb + h * p.ci_sh + beg;
   } else {
     static_assert(SPARSE || TN == kTileN, "dense kernel walks 64-key tiles");
@@ -145,7 +146,7 @@ __device__ __forceinline__ void prefill_item(const PrefillParams p, const int bi
   auto tile_k0 = [&](int it) __attribute__((always_inline)) -> int {
     if (!SPARSE) return it * TN;
     constexpr int PER = kTileN / TN;
-    return cols[it / PER] * kTileN + (it % PER) * TN;
+    return __builtin_amdgcn_readfirstlane(cols[it / PER]) * kTileN + (it % PER) * TN;
   };
   // The load is issued from inline assembly on purpose: the compiler then does
   // not know that LDS writes are in flight.  When it knows, it makes every
@@ -156,7 +157,8 @@ __device__ __forceinline__ void prefill_item(const PrefillParams p, const int bi
   // counted vmcnt waits below) followed by the workgroup barrier publishes a
   // tile.  M0 carries the LDS byte address of the 1 KiB slab.
   const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem);
-  auto dma16 = [&](const char* g, uint32_t slab) __attribute__((always_inline)) {
+  auto dma16 = [&](const char* g, uint32_t slab_u) __attribute__((always_inline)) {
+    const uint32_t slab = (uint32_t)__builtin_amdgcn_readfirstlane(slab_u);  // uniform by construction
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                  :
                  : "v"(g), "s"(slab)
@@ -548,7 +550,10 @@ int launch_one(const PrefillParams& p, hipStream_t s) {
   pp.n_items = (int)items;
   long long grid = items;
   if (!SPARSE) {
-    // one workgroup per CU is resident (LDS); more ids than that are walked in-kernel
+    // One workgroup per CU is resident (LDS); more ids than that are walked
+    // in-kernel.  (The sparse kernel keeps one launch per q tile: four small
+    // workgroups share a CU and cover each other's start-up, and walking ids
+    // in-kernel measured slower there.)
     const int cus = device_cu_count();
     if (cus > 0 && grid > cus) grid = cus;
   }

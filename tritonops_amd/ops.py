@@ -268,9 +268,11 @@ def _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, re
         a.split_tokens = 64
         a.block_idx, a.block_cnt = _ptr(block_idx), _ptr(block_cnt)
         a.block_idx_stride_b, a.block_idx_stride_h = bi_strides
-        a.max_blocks, a.block_size, a.split_blocks = int(max_blocks), _masks.BLOCK, int(split_blocks)
         a.window_local, a.window_global = window
         a.include_last_block = 1 if include_last else 0
+        a.max_blocks, a.block_size = int(max_blocks), _masks.BLOCK
+        a.split_blocks = int(split_blocks) if split_blocks else lib.mi_decode_choose_split_blocks(
+            B, Hkv, a.max_blocks + a.include_last_block, _NUM_CUS)
     nbytes = lib.mi_decode_workspace_bytes(C.byref(a))
     if nbytes == 0:
         raise _lib.MiAttnError(lib.mi_decode_validate(C.byref(a)), lib.mi_last_error().decode())
@@ -345,14 +347,13 @@ def flash_attention_sparse_decoding(q, k, v, cu_seq_lens, global_window_size=64,
         cap = n_sink + n_tail
         return _decode(q, k, v, None, lens, scale, None, None, return_lse, block_idx=idx, block_cnt=cnt,
                        bi_strides=(cap, 0), max_blocks=cap,
-                       split_blocks=split_blocks or max(1, min(8, cap)), window=(lw, gw))
+                       split_blocks=split_blocks or 0, window=(lw, gw))
     idx = block_indices.to(torch.int32).contiguous()
     if idx.dim() != 3 or idx.shape[0] != B or idx.shape[1] != Hkv:
         raise ValueError("block_indices must be [B, Hkv, n]")
     n = idx.shape[2]
     cnt = block_counts.to(torch.int32).contiguous() if block_counts is not None else None
     # the block of the newest token is appended (and de-duplicated) by the kernel
-    total = n + (1 if include_last_block else 0)
     return _decode(q, k, v, None, lens, scale, None, None, return_lse, block_idx=idx, block_cnt=cnt,
-                   bi_strides=(Hkv * n, n), max_blocks=n, split_blocks=split_blocks or max(1, min(8, total)),
+                   bi_strides=(Hkv * n, n), max_blocks=n, split_blocks=split_blocks or 0,
                    include_last=bool(include_last_block))
