@@ -138,6 +138,34 @@ def test_softmax_scale_and_extreme_scores():
         assert_close(got, ref, TOL)
 
 
+@pytest.mark.parametrize("slope", [0.5, 16.0, -16.0])
+@pytest.mark.parametrize("causal", [True, False])
+def test_scores_that_keep_growing_along_the_keys(slope, causal):
+    """s_ij = c * slope * j: every later half-tile beats the running reference
+    point of the row, mildly (slope 0.5: a few binades per 32 keys) or by more
+    than the fp32 exponent range (slope 16: exp2 overflows unless the reference
+    point is moved first); slope -16 is the mirror image (everything after the
+    first keys underflows).  Checked against fp32 softmax on the same inputs."""
+    import tritonops_amd as ta
+
+    B, H, S, D = 1, 2, 1100, 128
+    u = torch.full((D,), 0.125)
+    j = torch.arange(S, dtype=torch.float32)
+    k = (u[None, :] * (slope * j)[:, None]).to(torch.bfloat16)[None, None].expand(B, H, S, D).contiguous()
+    q = u.to(torch.bfloat16)[None, None, None, :].expand(B, H, S, D).contiguous()
+    v = randn((B, H, S, D), 5)
+    s = torch.einsum("bhid,bhjd->bhij", q.double(), k.double()) / math.sqrt(D)
+    if causal:
+        s = s.masked_fill(torch.arange(S)[None, :] > torch.arange(S)[:, None], float("-inf"))
+    ref = torch.einsum("bhij,bhjd->bhid", torch.softmax(s, -1), v.double()).float()
+    got, lse = ta.flash_attention(q.cuda(), k.cuda(), v.cuda(), causal=causal, return_lse=True)
+    assert torch.isfinite(got.float()).all()
+    assert_close(got, ref, TOL)
+    want_lse = (torch.logsumexp(s, -1) * orc.LOG2E).float()
+    rel = ((lse.cpu() - want_lse).abs() / want_lse.abs().clamp_min(1.0)).max().item()
+    assert rel <= 1e-3, rel
+
+
 def test_full_size_properties():
     """Size-independent checks at the benchmark shape B4 H32 S8192 D128: row 0
     equals v[0]; lse of zero-query rows; a head slice matches the oracle on a

@@ -220,15 +220,13 @@ __device__ __forceinline__ void prefill_item(const PrefillParams p, const int bi
 
   if constexpr (!SPARSE) {
     // ---- dense: software pipeline over HALF tiles (32 keys) inside each wave.
-    // A stalled MFMA blocks the vector ALU of its SIMD for every wave, so MFMA
-    // and softmax arithmetic only overlap when one wave's instruction stream
-    // interleaves them.  At position h the wave therefore runs, in ONE
-    // straight-line block, the 8 MFMAs of S[h+1] = K Q^T for the next half
-    // together with max / exp2 / convert of the current half S[h]; then
-    // (after the rare deferred rescale of O) the 8 MFMAs of O += V^T P^T for
-    // half h.  K of half h+1 must be in LDS while half h is being finished:
-    // tile t+1 has to be visible before position 2t+1, which the barrier at
-    // the top of tile t guarantees.
+    // MFMA and softmax arithmetic overlap best when one wave's instruction
+    // stream interleaves them, so at position h the wave runs two straight-line
+    // blocks: the 8 MFMAs of S[h+1] = K Q^T together with half of the exp2 /
+    // sum / convert work of S[h], then the 8 MFMAs of O += V^T P[h]^T together
+    // with the first half of that work for S[h+1].  K of half h+1 must be in LDS
+    // while half h is being finished: tile t+1 has to be visible before
+    // position 2t+1, which the barrier at the top of tile t guarantees.
     static_assert(TN == kTileN && NS >= 3, "pipelined dense path: 64-key tiles, >= 3 stages");
     int H_w = (len + 31) / 32;                        // halves this wave works on
     if (p.causal) H_w = min(H_w, q0w / 32 + 1);       // nothing above its own diagonal block
@@ -252,60 +250,70 @@ __device__ __forceinline__ void prefill_item(const PrefillParams p, const int bi
       }
     };
 
-    // The running-max update for the half in Sx, cut into pieces that are
-    // dropped behind successive MFMAs.  After piece 7: m is the reference max
-    // that the exponentials of Sx will use, l is on that scale, and O still
-    // has to be multiplied by alpha when grow is set.
-    float a0, a1, a2, a3, a4, mx, m_new, alpha;
-    bool grow;
-    auto max_piece = [&](int sl, const f32x16& Sx) __attribute__((always_inline)) {
-      if (sl == 1) {
-        a0 = fmaxf(fmaxf(Sx[0], Sx[1]), Sx[2]);
-        a1 = fmaxf(fmaxf(Sx[3], Sx[4]), Sx[5]);
-      } else if (sl == 2) {
-        a2 = fmaxf(fmaxf(Sx[6], Sx[7]), Sx[8]);
-        a3 = fmaxf(fmaxf(Sx[9], Sx[10]), Sx[11]);
-      } else if (sl == 3) {
-        a4 = fmaxf(fmaxf(Sx[12], Sx[13]), Sx[14]);
-        a0 = fmaxf(fmaxf(a0, a1), Sx[15]);
-      } else if (sl == 4) {
-        a2 = fmaxf(fmaxf(a2, a3), a4);
-        mx = fmaxf(a0, a2);
-      } else if (sl == 5) {
-        mx = max_with_other_half(mx);
-      } else if (sl == 6) {
-        m_new = fmaxf(m, mx * scale);
-        grow = __builtin_amdgcn_ballot_w64(m_new > m + kRescaleSlack) != 0;
-      } else if (sl == 7) {
-        const float m_next = grow ? m_new : m;
-        // a lane whose keys were all masked so far keeps m = -inf: factor 0 (l and O are 0)
-        alpha = fast_exp2(m - ((m_next == -INFINITY) ? 0.f : m_next));
-        l *= alpha;
-        m = m_next;
+    // Probabilities of a half are taken against the reference point m the row
+    // already has; m is only moved (exactly, to the true running maximum) when
+    // a lane's partial row sum of a half passes kRowSumLimit or is not finite.
+    // Any reference point gives the same o and lse, so the common path needs
+    // no row maximum at all: 7 vector instructions per pair of scores.
+    constexpr float kRowSumLimit = 4096.f;  // probabilities stay below 2^12: far inside bf16 / fp32 range
+    uint32_t Pb[2][8];  // packed probabilities of the half in S[0] / S[1]
+    float rsv[2];       // their partial row sums (this lane's 16 keys)
+    float e_p0, e_u1;   // first element done, second element scaled: carried between two slices
+    auto exp_first = [&](const f32x16& Sx, int i, float m_neg) __attribute__((always_inline)) {
+      e_p0 = fast_exp2(fmaf(Sx[2 * i], scale, m_neg));
+      e_u1 = fmaf(Sx[2 * i + 1], scale, m_neg);
+    };
+    auto exp_second = [&](int i, uint32_t (&Pd)[8], float& rs) __attribute__((always_inline)) {
+      const float p1 = fast_exp2(e_u1);
+      rs += e_p0 + p1;
+      Pd[i] = Elem<T>::pack2(e_p0, p1);
+    };
+    // rare: bring m to the exact running maximum including the half in Sx,
+    // rescale l and O, and redo the probabilities of that half
+    auto exact_fix = [&](const f32x16& Sx, uint32_t (&Pd)[8], float& rs) __attribute__((always_inline)) {
+      float mx = Sx[0];
+#pragma unroll
+      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, Sx[r]);
+      mx = max_with_other_half(mx);
+      const float m_new = fmaxf(m, mx * scale);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // no key seen yet: l and O are 0
+      const float alpha = fast_exp2(m - m_safe);
+      l *= alpha;
+#pragma unroll
+      for (int db = 0; db < G::NDB; ++db) O[db] *= alpha;
+      m = m_new;
+      rs = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float p0 = fast_exp2(fmaf(Sx[2 * i], scale, -m_safe));
+        const float p1 = fast_exp2(fmaf(Sx[2 * i + 1], scale, -m_safe));
+        rs += p0 + p1;
+        Pd[i] = Elem<T>::pack2(p0, p1);
       }
     };
 
-    // Position h.  Entry state: S[h&1] holds the scores of half h, m already
-    // includes them and O, l are on the scale of m; kf holds the first K
-    // fragments of half h+1.
-    //   block A: [MFMAs of S(h+1) = K Q^T] interleaved with [exp2 / sum / pack of S(h)]
-    //   block B: [MFMAs of O += V^T P(h)^T] interleaved with [max update for S(h+1)]
+    // Position h.  Entry state: S[h&1] holds the scores of half h and the
+    // probabilities of its first 8 keys per lane are done; kf holds the first
+    // K fragments of half h+1.
+    //   block A: [MFMAs of S(h+1) = K Q^T]      with [exp2 / sum / pack of the last 8 keys of S(h)]
+    //   check  : row sums sane? else exact_fix (rare)
+    //   block B: [MFMAs of O += V^T P(h)^T]    with [exp2 / sum / pack of the first 8 keys of S(h+1)]
+    // so every MFMA has three or four vector instructions behind it.
     // sched_barrier(0) after each slice pins the interleaving: one MFMA, the
-    // LDS reads for a slice four positions ahead, and a few VALU instructions.
+    // LDS reads for a slice four positions ahead, and those vector instructions.
     auto half_step = [&](auto j_c, int h) __attribute__((always_inline)) {
       constexpr int J = decltype(j_c)::value;  // h % (2 NS)
       if (h >= H_w) return;
-      const bool has_next = h + 1 < H_w;
       constexpr int TS = J / 2, KB = J & 1;    // stage of tile h/2, which half of it
       constexpr int KS = KB == 0 ? TS : (TS + 1) % NS;      // stage holding K of half h+1
       constexpr uint32_t KOFF = KS * TILEB, VOFF = TS * TILEB;
       constexpr uint32_t K2OFF = ((TS + 1) % NS) * TILEB;   // stage holding K of half h+2
       f32x16& Sc = S[KB];
       f32x16& Sn = S[KB ^ 1];
+      uint32_t (&Pc)[8] = Pb[KB];
+      uint32_t (&Pn)[8] = Pb[KB ^ 1];
       const float m_neg = (m == -INFINITY) ? 0.f : -m;
-      uint32_t P[8];
       i32x4 vf[G::NDB];
-      float rs = 0.f;
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         if (c < G::KSTEPS) {
@@ -314,40 +322,37 @@ __device__ __forceinline__ void prefill_item(const PrefillParams p, const int bi
           if (c + KR < G::KSTEPS) kf[c % KR] = fr.load_k(KOFF, KB ^ 1, c + KR);
         }
         if (c >= 8 - G::NDB) vf[c - (8 - G::NDB)] = fr.load_v(VOFF, 2 * KB, c - (8 - G::NDB));
-        const float p0 = fast_exp2(fmaf(Sc[2 * c], scale, m_neg));
-        const float p1 = fast_exp2(fmaf(Sc[2 * c + 1], scale, m_neg));
-        rs += p0 + p1;
-        P[c] = Elem<T>::pack2(p0, p1);
+        if ((c & 1) == 0)
+          exp_first(Sc, 4 + c / 2, m_neg);
+        else
+          exp_second(4 + c / 2, Pc, rsv[KB]);
         __builtin_amdgcn_sched_barrier(0);
       }
-      l += rs;
       // keep the exponentials in this block (they would otherwise sink below
       // the branches that follow, away from the MFMAs they are meant to overlap)
-      asm volatile("" : "+v"(P[0]), "+v"(P[1]), "+v"(P[2]), "+v"(P[3]), "+v"(P[4]), "+v"(P[5]), "+v"(P[6]), "+v"(P[7]), "+v"(l));
+      asm volatile("" : "+v"(Pc[4]), "+v"(Pc[5]), "+v"(Pc[6]), "+v"(Pc[7]), "+v"(rsv[KB]));
+      if (__builtin_amdgcn_ballot_w64(!(rsv[KB] <= kRowSumLimit)) != 0) exact_fix(Sc, Pc, rsv[KB]);
+      l += rsv[KB];
       mask_half(h + 1, Sn);
-      const float m_keep = m, l_keep = l;
+      const float m_neg2 = (m == -INFINITY) ? 0.f : -m;
+      rsv[KB ^ 1] = 0.f;
 #pragma unroll
       for (int sl = 0; sl < 8; ++sl) {
         if (sl < 2 * G::NDB) {
           const int kk = sl / G::NDB, db = sl % G::NDB;
-          const i32x4 pf = {(int)P[4 * kk], (int)P[4 * kk + 1], (int)P[4 * kk + 2], (int)P[4 * kk + 3]};
+          const i32x4 pf = {(int)Pc[4 * kk], (int)Pc[4 * kk + 1], (int)Pc[4 * kk + 2], (int)Pc[4 * kk + 3]};
           O[db] = Elem<T>::mfma(vf[db], pf, O[db]);
           if (kk == 0) vf[db] = fr.load_v(VOFF, 2 * KB + 1, db);
         }
         if (sl >= 4 && sl - 4 < KR) kf[sl - 4] = fr.load_k(K2OFF, KB, sl - 4);
-        max_piece(sl, Sn);
+        // (for the last half of a wave Sn holds scores of stale LDS contents: the results are never used)
+        if ((sl & 1) == 0)
+          exp_first(Sn, sl / 2, m_neg2);
+        else
+          exp_second(sl / 2, Pn, rsv[KB ^ 1]);
         __builtin_amdgcn_sched_barrier(0);
       }
-      // The last half of a wave scored stale LDS contents above (no half h+1
-      // exists); drop that update.
-      m = has_next ? m : m_keep;
-      l = has_next ? l : l_keep;
-      asm volatile("" : "+v"(m), "+v"(l));
-      // rare: the reference max moved, bring O to the new scale
-      if (grow && has_next) {
-#pragma unroll
-        for (int db = 0; db < G::NDB; ++db) O[db] *= alpha;
-      }
+      asm volatile("" : "+v"(Pn[0]), "+v"(Pn[1]), "+v"(Pn[2]), "+v"(Pn[3]), "+v"(rsv[KB ^ 1]));
     };
 
     // tile t: barrier (tile t+1 visible, stage of tile t-1 free), refill, two halves
@@ -379,14 +384,20 @@ __device__ __forceinline__ void prefill_item(const PrefillParams p, const int bi
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __syncthreads();
     if (H_w > 0) {
-      // scores and running max of half 0, then the first fragments of half 1
+      // scores of half 0, its exact row maximum as the first reference point,
+      // the probabilities of its first 8 keys, then the first fragments of half 1
       f32x16 acc = (f32x16){0};
 #pragma unroll
       for (int c = 0; c < G::KSTEPS; ++c) acc = Elem<T>::mfma(fr.load_k(0u, 0, c), Qf[c], acc);
       S[0] = acc;
       mask_half(0, S[0]);
+      exact_fix(S[0], Pb[0], rsv[0]);
+      rsv[0] = 0.f;
 #pragma unroll
-      for (int sl = 1; sl < 8; ++sl) max_piece(sl, S[0]);
+      for (int i = 0; i < 4; ++i) {
+        exp_first(S[0], i, (m == -INFINITY) ? 0.f : -m);
+        exp_second(i, Pb[0], rsv[0]);
+      }
 #pragma unroll
       for (int c = 0; c < KR; ++c) kf[c] = fr.load_k(0u, 1, c);
     }
