@@ -152,6 +152,24 @@ def run_decode(steps, warmup):
     a.workspace, a.workspace_bytes = ws.data_ptr(), nbytes
     k_split = _event_ms(3, a, steps, warmup)
     k_merge = _event_ms(4, a, steps, warmup)
+    # same cache as a pool of shuffled 64-token pages [pages, Hkv, 64, D] behind a page table
+    ps = 64
+    npg = L // ps
+    perm = torch.randperm(B * npg, generator=torch.Generator().manual_seed(3)).cuda()
+    table = perm.view(B, npg).to(torch.int32)
+    pools = []
+    for t in (kc, vc):
+        pool = torch.empty((B * npg, Hkv, ps, D), device="cuda", dtype=t.dtype)
+        pool[perm] = t.view(B, Hkv, npg, ps, D).permute(0, 2, 1, 3, 4).reshape(B * npg, Hkv, ps, D)
+        pools.append(pool.transpose(1, 2))
+    kp, vp = pools
+    a.k, a.v = kp.data_ptr(), vp.data_ptr()
+    a.k_stride_b, a.k_stride_s, a.k_stride_h = kp.stride(0), kp.stride(1), kp.stride(2)
+    a.v_stride_b, a.v_stride_s, a.v_stride_h = vp.stride(0), vp.stride(1), vp.stride(2)
+    a.kv_layout, a.page_size = _lib.MI_KV_PAGED, ps
+    a.page_table, a.page_table_stride_b = table.data_ptr(), table.stride(0)
+    k_paged = _event_ms(3, a, steps, warmup)
+    del pools, kp, vp
     nbytes_alg = float(lens.sum().item()) * Hkv * 2 * D * 2 + B * Hq * D * 2 * 2
     return {
         "name": "gqa_decode", "ms_per_step": ms, "kernel_ms": k_split, "merge_kernel_ms": k_merge,
@@ -159,7 +177,9 @@ def run_decode(steps, warmup):
         "roofline": {"bound": "hbm", "achieved": nbytes_alg / (k_split * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "kernel": "decode_splitkv_kernel<bf16,128>"},
         "config": {"workload": "GQA decode bf16 B=64 Hq=32 Hkv=8 KV<=32768 (lens U[16384,32768]) D=128, split-KV + LSE merge",
-                   "bytes_per_step": nbytes_alg, "split_tokens": int(a.split_tokens)},
+                   "bytes_per_step": nbytes_alg, "split_tokens": int(a.split_tokens),
+                   "paged_cache_kernel_ms": k_paged,
+                   "paged_cache_note": "same launch over a pool of shuffled 64-token pages behind a page table"},
     }
 
 
@@ -307,8 +327,8 @@ def cpu_baseline(name):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=40)
+    ap.add_argument("--warmup", type=int, default=15)
     ap.add_argument("--workload", default="all", choices=["all"] + list(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true",

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define MI_ATTN_ABI_VERSION 1
+#define MI_ATTN_ABI_VERSION 2
 
 /* KV tile edge (tokens) of the prefill kernels and block edge of the block
  * sparse layouts; fixed at build time. */
@@ -179,6 +179,20 @@ int mi_attn_fwd_blocksparse(const mi_attn_sparse_args *args, void *stream);
  * :391-396:  allowed(k) = k < window_global or k >= seq_len - window_local
  * (pass -1/-1 to disable).
  */
+/* Where token t of sequence b lives in k / v (element strides as given):
+ *   MI_KV_BATCHED  k + b*k_stride_b + t*k_stride_s            ([batch, max_seqlen, heads_kv, D] view; the
+ *                  layout flash_attention_decoding takes, flash_attn_decoding.py:283-290)
+ *   MI_KV_PACKED   k + (cu_seqlens[b] + t)*k_stride_s          (one [total_tokens, heads_kv, D] buffer, the
+ *                  layout the reference's decode oracle consumes, flash_attn_decoding.py:357-359;
+ *                  needs cu_seqlens, k_stride_b is ignored)
+ *   MI_KV_PAGED    k + page_table[b][t / page_size]*k_stride_b + (t % page_size)*k_stride_s
+ *                  (a pool of pages [num_pages, page_size, heads_kv, D]; k_stride_b is the page stride).
+ * No counterpart of the paged form exists in the reference; it is the cache
+ * layout of a serving loop around this call. */
+#define MI_KV_BATCHED 0
+#define MI_KV_PACKED 1
+#define MI_KV_PAGED 2
+
 typedef struct mi_decode_args {
   uint32_t struct_size;
   int32_t dtype;
@@ -211,6 +225,12 @@ typedef struct mi_decode_args {
   int32_t window_global;         /* tokens, or -1                              */
   int32_t include_last_block;    /* 1: also attend the block holding token     */
                                  /* seq_len-1 (listed or not, counted once)    */
+  /* KV-cache layout (see MI_KV_* above) */
+  int32_t kv_layout;             /* MI_KV_BATCHED, MI_KV_PACKED or MI_KV_PAGED */
+  int32_t page_size;             /* paged: tokens per page, multiple of 32     */
+  const int32_t *page_table;     /* paged: device; physical page of logical    */
+                                 /* page p of sequence b at [b*stride_b + p]   */
+  int64_t page_table_stride_b;
 } mi_decode_args;
 
 /* Number of pass-1 chunks per sequence for these arguments (host only). */

@@ -27,7 +27,7 @@ def test_every_declared_symbol_is_exported(lib):
     assert declared == set(_lib.EXPORTS), "ctypes table and header disagree: %s" % (declared ^ set(_lib.EXPORTS))
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.mi_abi_version() == 1
+    assert lib.mi_abi_version() == _lib.MI_ATTN_ABI_VERSION == 2
 
 
 def test_struct_layout_matches_the_c_compiler(tmp_path):
@@ -35,13 +35,13 @@ def test_struct_layout_matches_the_c_compiler(tmp_path):
     src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "mi_attn.h"\nint main(){printf("%zu %zu %zu %zu %zu %zu\\n",'
                    "sizeof(mi_attn_fwd_args),sizeof(mi_attn_sparse_args),sizeof(mi_decode_args),"
                    "offsetof(mi_attn_fwd_args,scale_log2),offsetof(mi_attn_sparse_args,scale_log2),"
-                   "offsetof(mi_decode_args,window_global));return 0;}\n")
+                   "offsetof(mi_decode_args,page_table));return 0;}\n")
     exe = tmp_path / "sz"
     subprocess.check_call(["gcc", "-std=c99", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
     got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
     want = [C.sizeof(_lib.AttnFwdArgs), C.sizeof(_lib.AttnSparseArgs), C.sizeof(_lib.DecodeArgs),
             _lib.AttnFwdArgs.scale_log2.offset, _lib.AttnSparseArgs.scale_log2.offset,
-            _lib.DecodeArgs.window_global.offset]
+            _lib.DecodeArgs.page_table.offset]
     assert got == want
 
 
@@ -174,6 +174,26 @@ def test_decode_geometry_and_validation(lib):
     assert lib.mi_decode_validate(C.byref(a)) == 0
     a.block_size = 32
     assert lib.mi_status_name(lib.mi_decode_validate(C.byref(a))).decode() == "MI_ERR_SPARSE_LAYOUT"
+
+
+def test_decode_kv_layout_validation(lib):
+    a = _good_decode()
+    a.kv_layout = 7
+    assert lib.mi_status_name(lib.mi_decode_validate(C.byref(a))).decode() == "MI_ERR_SHAPE"
+    a = _good_decode()
+    a.kv_layout = 2                                   # paged
+    a.page_size, a.page_table = 48, 0x6000
+    assert lib.mi_status_name(lib.mi_decode_validate(C.byref(a))).decode() == "MI_ERR_SHAPE"   # not a multiple of 32
+    a.page_size, a.page_table = 64, None
+    assert lib.mi_status_name(lib.mi_decode_validate(C.byref(a))).decode() == "MI_ERR_NULL_POINTER"
+    a.page_table = 0x6000
+    assert lib.mi_decode_validate(C.byref(a)) == 0
+    a = _good_decode()
+    a.kv_layout = 1                                   # packed: offsets come from cu_seqlens
+    if a.cu_seqlens:
+        assert lib.mi_decode_validate(C.byref(a)) == 0
+        a.seq_lens, a.cu_seqlens = a.cu_seqlens, None
+    assert lib.mi_status_name(lib.mi_decode_validate(C.byref(a))).decode() == "MI_ERR_NULL_POINTER"
 
 
 def test_split_heuristic(lib):

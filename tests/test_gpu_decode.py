@@ -160,3 +160,90 @@ def test_last_block_listed_and_implicit_counts_once():
                                              block_indices=idx.cuda(), block_counts=cnt.cuda(),
                                              include_last_block=False)
     assert_close(got, no_last, TOL)
+
+
+def _paginate(k, v, lens, page_size, seed):
+    """Scatter a [B,L,Hkv,D] cache into a shuffled page pool; returns pools and
+    the page table (unused entries point at a poisoned page)."""
+    B, L, Hkv, D = k.shape
+    pages_per_seq = (L + page_size - 1) // page_size
+    need = [(int(n) + page_size - 1) // page_size for n in lens]
+    total = sum(need) + 1
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(total - 1, generator=g) + 1          # page 0 stays poisoned
+    kp = torch.full((total, page_size, Hkv, D), float("nan"), dtype=k.dtype)
+    vp = torch.full((total, page_size, Hkv, D), float("nan"), dtype=v.dtype)
+    table = torch.zeros((B, pages_per_seq), dtype=torch.int32)
+    nxt = 0
+    for b in range(B):
+        for p in range(need[b]):
+            phys = int(perm[nxt]); nxt += 1
+            table[b, p] = phys
+            rows = slice(p * page_size, min((p + 1) * page_size, L))
+            n = rows.stop - rows.start
+            kp[phys, :n] = k[b, rows]
+            vp[phys, :n] = v[b, rows]
+            # rows of the last page beyond the sequence hold finite junk (they are masked, not skipped)
+            kp[phys, n:] = 7.0
+            vp[phys, n:] = -7.0
+    return kp, vp, table
+
+
+@pytest.mark.parametrize("page_size", [32, 64, 256])
+def test_paged_cache_is_bit_identical_to_batched(page_size):
+    """The page table only changes where a tile is fetched from: same kernel,
+    same order of operations, so the outputs must be equal bit for bit."""
+    import tritonops_amd as ta
+
+    lens = torch.tensor([777, 2049, 64, 0, 1, 33, 4096], dtype=torch.int32)
+    B, Hq, Hkv, D = len(lens), 8, 2, 128
+    L = int(lens.max())
+    q = randn((B, Hq, D), 21)
+    k, v = _kv(B, L, Hkv, D, torch.bfloat16, 22)
+    ref, ref_lse = ta.flash_attention_decoding(q.cuda(), k.cuda(), v.cuda(), None, seq_lens=lens.cuda(),
+                                               split_tokens=256, return_lse=True)
+    kp, vp, table = _paginate(k, v, lens, page_size, 5)
+    got, lse = ta.flash_attention_decoding(q.cuda(), kp.cuda(), vp.cuda(), None, seq_lens=lens.cuda(),
+                                           split_tokens=256, return_lse=True, kv_layout="paged",
+                                           page_table=table.cuda(), max_seq_len=L)
+    assert torch.equal(got, ref) and torch.equal(lse, ref_lse)
+    want = orc.flash_attn_decoding_torch(q, k, v, lens, faithful=False)
+    assert_close(got, want, TOL)
+    # block-list form over the same pages
+    idx = torch.zeros((B, Hkv, 6), dtype=torch.int32)
+    cnt = torch.zeros((B, Hkv), dtype=torch.int32)
+    for b, n in enumerate(lens):
+        nblk = (int(n) + 63) // 64
+        for h in range(Hkv):
+            c = min(6, nblk)
+            pick = torch.randperm(max(nblk, 1), generator=torch.Generator().manual_seed(b * 7 + h))[:c]
+            idx[b, h, :c] = torch.sort(pick).values.to(torch.int32)
+            cnt[b, h] = c
+    a = ta.flash_attention_sparse_decoding(q.cuda(), k.cuda(), v.cuda(), None, seq_lens=lens.cuda(),
+                                           block_indices=idx.cuda(), block_counts=cnt.cuda())
+    b_ = ta.flash_attention_sparse_decoding(q.cuda(), kp.cuda(), vp.cuda(), None, seq_lens=lens.cuda(),
+                                            block_indices=idx.cuda(), block_counts=cnt.cuda(),
+                                            kv_layout="paged", page_table=table.cuda())
+    assert torch.equal(a, b_)
+    assert torch.isfinite(a.float()).all()
+
+
+def test_packed_cache_matches_batched_and_reference_oracle_layout():
+    """k, v as one [1,T,Hkv,D] buffer addressed through cu_seq_lens — the layout
+    the reference's decode oracle takes (flash_attn_decoding.py:357-359)."""
+    import tritonops_amd as ta
+
+    lens = torch.tensor([512, 2049, 1, 0, 65, 300], dtype=torch.int32)
+    B, Hq, Hkv, D = len(lens), 6, 2, 96
+    L = int(lens.max())
+    q = randn((B, Hq, D), 31, torch.float16)
+    k, v = _kv(B, L, Hkv, D, torch.float16, 32)
+    cu = cu_from(lens)
+    kpk = torch.cat([k[b, :int(n)] for b, n in enumerate(lens)])[None]
+    vpk = torch.cat([v[b, :int(n)] for b, n in enumerate(lens)])[None]
+    ref = ta.flash_attention_decoding(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), split_tokens=128)
+    got = ta.flash_attention_decoding(q.cuda(), kpk.cuda(), vpk.cuda(), cu.cuda(), split_tokens=128,
+                                      kv_layout="packed", max_seq_len=L)
+    assert torch.equal(got, ref)
+    want = orc.flash_attn_decoding_torch(q, k, v, lens, faithful=False)
+    assert_close(got, want, TOL)

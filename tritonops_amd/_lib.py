@@ -9,7 +9,8 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmi_attn.so")
 
-MI_ATTN_ABI_VERSION = 1
+MI_ATTN_ABI_VERSION = 2
+MI_KV_BATCHED, MI_KV_PACKED, MI_KV_PAGED = 0, 1, 2
 MI_ATTN_BLOCK = 64
 MI_DTYPE_BF16 = 0
 MI_DTYPE_F16 = 1
@@ -88,6 +89,8 @@ class DecodeArgs(C.Structure):
         ("max_blocks", _i32), ("block_size", _i32), ("split_blocks", _i32),
         ("window_local", _i32), ("window_global", _i32),
         ("include_last_block", _i32),
+        ("kv_layout", _i32), ("page_size", _i32),
+        ("page_table", _vp), ("page_table_stride_b", _i64),
     ]
 
 

@@ -105,6 +105,8 @@ void fill_decode(const mi_decode_args* a, mi::DecodeParams& p) {
   p.win_global = a->block_idx ? a->window_global : -1;
   p.add_last = (a->block_idx && a->include_last_block) ? 1 : 0;
   if (!a->block_idx) { p.max_blocks = 0; p.split_blocks = 1; }
+  p.kv_layout = a->kv_layout; p.page_size = a->page_size;
+  p.page_table = a->page_table; p.pt_sb = a->page_table_stride_b;
 }
 
 int launch_status(int hip_err, const char* what) {
@@ -218,6 +220,11 @@ static int decode_validate_shape(const mi_decode_args* a) {
     if (a->split_tokens <= 0 || a->split_tokens % 64 != 0)
       return fail(MI_ERR_WORKSPACE, "split_tokens %d must be a positive multiple of 64", a->split_tokens);
   }
+  if (a->kv_layout != MI_KV_BATCHED && a->kv_layout != MI_KV_PACKED && a->kv_layout != MI_KV_PAGED)
+    return fail(MI_ERR_SHAPE, "kv_layout %d is not MI_KV_BATCHED / MI_KV_PACKED / MI_KV_PAGED", a->kv_layout);
+  if (a->kv_layout == MI_KV_PAGED && (a->page_size <= 0 || a->page_size % 32 != 0 || a->page_table_stride_b < 0))
+    return fail(MI_ERR_SHAPE, "paged KV needs page_size a positive multiple of 32 (got %d) and a page table stride >= 0",
+                a->page_size);
   if (decode_splits(a) > 65535) return fail(MI_ERR_WORKSPACE, "more than 65535 splits per sequence");
   if (a->heads_kv > 65535 || a->batch > 65535 || a->heads_q > 0x7fffffff / 2)
     return fail(MI_ERR_SHAPE, "batch / head count exceeds the launch grid limits");
@@ -272,6 +279,10 @@ int mi_decode_validate(const mi_decode_args* a) {
     return fail(MI_ERR_ALIGNMENT, "q, k and v must be 16-byte aligned");
   if ((a->seq_lens == nullptr) == (a->cu_seqlens == nullptr))
     return fail(MI_ERR_NULL_POINTER, "exactly one of seq_lens / cu_seqlens must be non-NULL");
+  if (a->kv_layout == MI_KV_PACKED && !a->cu_seqlens)
+    return fail(MI_ERR_NULL_POINTER, "packed KV takes the row offsets from cu_seqlens");
+  if (a->kv_layout == MI_KV_PAGED && !a->page_table)
+    return fail(MI_ERR_NULL_POINTER, "paged KV needs page_table");
   const int64_t s[] = {a->q_stride_b, a->q_stride_h, a->k_stride_b, a->k_stride_s, a->k_stride_h,
                        a->v_stride_b, a->v_stride_s, a->v_stride_h};
   for (int64_t x : s)

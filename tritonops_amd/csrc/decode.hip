@@ -72,8 +72,23 @@ decode_splitkv_kernel(const DecodeParams p) {
     return blk * 64 + (i & 1) * kDecTile;
   };
 
-  const T* kp = reinterpret_cast<const T*>(p.k) + b * p.k_sb + kvh * p.k_sh;
-  const T* vp = reinterpret_cast<const T*>(p.v) + b * p.v_sb + kvh * p.v_sh;
+  // Start of this sequence's rows: batch stride, row offset cu[b] of a packed
+  // buffer, or (paged) the pool itself with the page looked up per tile.
+  const int64_t seq0 = p.kv_layout == 1 ? (int64_t)p.cu[b] : 0;
+  const int64_t bsel = p.kv_layout == 0 ? b : 0;
+  const T* kp = reinterpret_cast<const T*>(p.k) + bsel * p.k_sb + seq0 * p.k_ss + kvh * p.k_sh;
+  const T* vp = reinterpret_cast<const T*>(p.v) + bsel * p.v_sb + seq0 * p.v_ss + kvh * p.v_sh;
+  const bool paged = p.kv_layout == 2;
+  const int32_t* ptab = paged ? p.page_table + b * p.pt_sb : nullptr;
+  // Paged: a 32-token tile never straddles a page (page_size % 32 == 0).  The
+  // returned element offset moves token `tb` of the flat addressing below onto
+  // its place in the physical page.
+  auto page_shift = [&](int tb, int64_t page_stride, int64_t row_stride) -> int64_t {
+    if (!paged) return 0;
+    const int lp = tb / p.page_size;
+    const int64_t phys = ptab[lp];
+    return phys * page_stride - (int64_t)lp * p.page_size * row_stride;
+  };
 
   F lc;
   lc.init(lane);
@@ -96,15 +111,25 @@ decode_splitkv_kernel(const DecodeParams p) {
   float m = -INFINITY, l = 0.f;
 
   i32x4 kreg[LOADS], vreg[LOADS];
-  auto gload = [&](int base) {
+  // First token a tile is fetched from.  A tile that is masked as a whole (a
+  // dropped duplicate, base -1, or the second half of the last block when the
+  // sequence ends in its first half) is fetched from the tile of the last
+  // token instead, so that no row outside [0, len) and no page beyond the
+  // sequence is ever touched.
+  const int last_tile = ((len - 1) / kDecTile) * kDecTile;
+  auto addr_base = [&](int base) -> int { return min(max(base, 0), last_tile); };
+  // kshift / vshift: page_shift() of the tile (0 unless paged)
+  auto gload = [&](int base, int64_t kshift, int64_t vshift) {
+    const int tb = addr_base(base);
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       const int idx = lane + i * 64;
       if (NCHUNK % 64 == 0 || idx < NCHUNK) {
         const int row = idx / G::NCH, ch = idx % G::NCH;
-        const int64_t kr = max(0, min(base + row, len - 1));
-        kreg[i] = *reinterpret_cast<const i32x4*>(kp + kr * p.k_ss + ch * 8);
-        vreg[i] = *reinterpret_cast<const i32x4*>(vp + kr * p.v_ss + ch * 8);
+        // rows past the end re-read the last token (same tile, hence same page)
+        const int64_t kr = min(tb + row, len - 1);
+        kreg[i] = *reinterpret_cast<const i32x4*>(kp + kshift + kr * p.k_ss + ch * 8);
+        vreg[i] = *reinterpret_cast<const i32x4*>(vp + vshift + kr * p.v_ss + ch * 8);
       }
     }
   };
@@ -121,12 +146,26 @@ decode_splitkv_kernel(const DecodeParams p) {
   };
 
   const int wl = p.win_local, wg = p.win_global;
-  gload(tile_base(0));
+  // tile bases and page look-ups run one tile ahead of the loads that use
+  // them, which run one tile ahead of the compute
+  int base_cur = tile_base(0);
+  {
+    const int tb = addr_base(base_cur);
+    gload(base_cur, page_shift(tb, p.k_sb, p.k_ss), page_shift(tb, p.v_sb, p.v_ss));
+  }
+  int base_nxt = n_tiles > 1 ? tile_base(1) : 0;
+  int64_t ks_nxt = page_shift(addr_base(base_nxt), p.k_sb, p.k_ss), vs_nxt = page_shift(addr_base(base_nxt), p.v_sb, p.v_ss);
   lstore();
   for (int it = 0; it < n_tiles; ++it) {
-    const int base = tile_base(it);
+    const int base = base_cur;
     const bool more = it + 1 < n_tiles;
-    if (more) gload(tile_base(it + 1));
+    if (more) gload(base_nxt, ks_nxt, vs_nxt);
+    base_cur = base_nxt;
+    if (it + 2 < n_tiles) {
+      base_nxt = tile_base(it + 2);
+      ks_nxt = page_shift(addr_base(base_nxt), p.k_sb, p.k_ss);
+      vs_nxt = page_shift(addr_base(base_nxt), p.v_sb, p.v_ss);
+    }
     bool need_mask = base + kDecTile > len || base < 0;
     if (wl >= 0) need_mask = need_mask || !((base + kDecTile - 1 < wg) || (base >= len - wl));
     auto allowed = [&](int key_in_tile) -> bool {

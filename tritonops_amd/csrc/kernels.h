@@ -51,6 +51,11 @@ struct DecodeParams {
   int32_t max_blocks, split_blocks;
   int32_t win_local, win_global;
   int32_t add_last;  // implicit extra entry: the block of token len-1
+  // KV-cache layout: 0 batched, 1 packed (rows of sequence b start at cu[b]), 2 paged
+  int32_t kv_layout;
+  int32_t page_size;
+  const int32_t* page_table;
+  int64_t pt_sb;
 };
 
 // dtype: 0 bf16, 1 f16.  head_dim in {64, 96, 128}.  Return hipError_t as int.

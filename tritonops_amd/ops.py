@@ -233,8 +233,8 @@ def flash_attn_sparse_triton(q, k, v, cu_seqlens, softmax_scale=None, local_wind
 
 def _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, return_lse,
             block_idx=None, block_cnt=None, bi_strides=(0, 0), max_blocks=0, split_blocks=0,
-            window=(-1, -1), include_last=False):
-    _require_gpu(q, k, v, cu_seq_lens, seq_lens)
+            window=(-1, -1), include_last=False, kv_layout="batched", page_table=None, page_size=0):
+    _require_gpu(q, k, v, cu_seq_lens, seq_lens, page_table)
     lib = _lib.load()
     q, k, v = _inner_contig(q), _inner_contig(k), _inner_contig(v)
     B, Hq, D = q.shape
@@ -258,8 +258,32 @@ def _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, re
         cu_seq_lens = cu_seq_lens.to(torch.int32)
         a.seq_lens, a.cu_seqlens = None, _ptr(cu_seq_lens)
     a.batch, a.heads_q, a.heads_kv, a.head_dim = B, Hq, Hkv, D
-    # k.shape[1] bounds every length, so no host sync is needed for the grid
-    a.max_seqlen = int(k.shape[1] if max_seq_len is None else min(max_seq_len, k.shape[1]))
+    if kv_layout == "batched":
+        if k.shape[0] != B:
+            raise ValueError("k, v must be [B, maxL, Hkv, D] (pass kv_layout='packed' for a [1, T, Hkv, D] buffer)")
+        a.kv_layout = _lib.MI_KV_BATCHED
+        bound = k.shape[1]      # bounds every length, so no host sync is needed for the grid
+    elif kv_layout == "packed":
+        if k.shape[0] != 1 or cu_seq_lens is None:
+            raise ValueError("packed KV is one [1, T, Hkv, D] buffer addressed through cu_seq_lens")
+        a.kv_layout = _lib.MI_KV_PACKED
+        bound = k.shape[1]
+    elif kv_layout == "paged":
+        # k, v: page pools [num_pages, page_size, Hkv, D]; page_table [B, max_pages] int32
+        if page_table is None or page_table.dim() != 2 or page_table.shape[0] != B:
+            raise ValueError("paged KV needs page_table [B, max_pages]")
+        page_table = page_table.to(torch.int32)
+        if page_table.stride(1) != 1:
+            page_table = page_table.contiguous()
+        page_size = int(page_size or k.shape[1])
+        if page_size != k.shape[1] or page_size % 32 != 0:
+            raise ValueError("page_size must equal k.shape[1] and be a multiple of 32")
+        a.kv_layout, a.page_size = _lib.MI_KV_PAGED, page_size
+        a.page_table, a.page_table_stride_b = _ptr(page_table), page_table.stride(0)
+        bound = page_table.shape[1] * page_size
+    else:
+        raise ValueError("kv_layout must be 'batched', 'packed' or 'paged'")
+    a.max_seqlen = int(bound if max_seq_len is None else min(max_seq_len, bound))
     a.scale_log2 = float(scale) * LOG2E
     if block_idx is None:
         a.split_tokens = int(split_tokens) if split_tokens else lib.mi_decode_choose_split_tokens(
@@ -283,7 +307,8 @@ def _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, re
 
 
 def flash_attention_decoding(q, k, v, cu_seq_lens, qk_scale=None, *, seq_lens=None, max_seq_len=None,
-                             split_tokens=None, return_lse=False):
+                             split_tokens=None, return_lse=False, kv_layout="batched", page_table=None,
+                             page_size=None):
     """Single-query decoding, split-KV + LSE merge.
 
     Contract of flash_attention_decoding in
@@ -292,17 +317,24 @@ def flash_attention_decoding(q, k, v, cu_seq_lens, qk_scale=None, *, seq_lens=No
     cu_seq_lens [B+1] supplies only the lengths (:46-48); `qk_scale` natural
     base, default D^-0.5 (:236-237).  Returns o [B,Hq,D]; rows with length 0
     are zero.  Extensions: `seq_lens` [B] instead of cu_seq_lens, `max_seq_len`
-    and `split_tokens` to size the launch, `return_lse` (base-2, [B,Hq]).
+    and `split_tokens` to size the launch, `return_lse` (base-2, [B,Hq]), and
+    two more KV-cache layouts: kv_layout="packed" — k, v [1,T,Hkv,D] with
+    sequence b in rows cu_seq_lens[b]:cu_seq_lens[b+1], what the reference's
+    decode oracle consumes (:357-359); kv_layout="paged" — k, v are page pools
+    [num_pages, page_size, Hkv, D] and page_table [B, max_pages] int32 maps a
+    sequence's logical pages to pool pages (page_size a multiple of 32).
     """
     if (cu_seq_lens is None) == (seq_lens is None):
         raise ValueError("give exactly one of cu_seq_lens / seq_lens")
     scale = q.shape[-1] ** -0.5 if qk_scale is None else qk_scale
-    return _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, return_lse)
+    return _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, return_lse,
+                   kv_layout=kv_layout, page_table=page_table, page_size=page_size or 0)
 
 
 def flash_attention_sparse_decoding(q, k, v, cu_seq_lens, global_window_size=64, local_window_size=64, *,
                                     seq_lens=None, block_indices=None, block_counts=None, block_size=64,
-                                    include_last_block=True, split_blocks=None, return_lse=False):
+                                    include_last_block=True, split_blocks=None, return_lse=False,
+                                    kv_layout="batched", page_table=None, page_size=None):
     """Sparse single-query decoding.
 
     Window form — contract of flash_attention_sparse_decoding in
@@ -315,7 +347,12 @@ def flash_attention_sparse_decoding(q, k, v, cu_seq_lens, global_window_size=64,
     by its query heads; `block_counts` [B,Hkv] optionally gives the number of
     valid entries; with `include_last_block` the block holding the newest
     token is added if absent.  Tokens >= len are masked.
+    Both forms also read a paged cache (kv_layout="paged", page_table,
+    page_size as in flash_attention_decoding).
     """
+    if kv_layout not in ("batched", "paged"):
+        raise ValueError("sparse decoding reads a 'batched' or a 'paged' cache")
+    layout = dict(kv_layout=kv_layout, page_table=page_table, page_size=page_size or 0)
     if (cu_seq_lens is None) == (seq_lens is None):
         raise ValueError("give exactly one of cu_seq_lens / seq_lens")
     if block_size != _masks.BLOCK:
@@ -347,7 +384,7 @@ def flash_attention_sparse_decoding(q, k, v, cu_seq_lens, global_window_size=64,
         cap = n_sink + n_tail
         return _decode(q, k, v, None, lens, scale, None, None, return_lse, block_idx=idx, block_cnt=cnt,
                        bi_strides=(cap, 0), max_blocks=cap,
-                       split_blocks=split_blocks or 0, window=(lw, gw))
+                       split_blocks=split_blocks or 0, window=(lw, gw), **layout)
     idx = block_indices.to(torch.int32).contiguous()
     if idx.dim() != 3 or idx.shape[0] != B or idx.shape[1] != Hkv:
         raise ValueError("block_indices must be [B, Hkv, n]")
@@ -356,4 +393,4 @@ def flash_attention_sparse_decoding(q, k, v, cu_seq_lens, global_window_size=64,
     # the block of the newest token is appended (and de-duplicated) by the kernel
     return _decode(q, k, v, None, lens, scale, None, None, return_lse, block_idx=idx, block_cnt=cnt,
                    bi_strides=(Hkv * n, n), max_blocks=n, split_blocks=split_blocks or 0,
-                   include_last=bool(include_last_block))
+                   include_last=bool(include_last_block), **layout)
