@@ -100,6 +100,44 @@ typedef struct mi_attn_fwd_args {
 int mi_attn_fwd(const mi_attn_fwd_args *args, void *stream);
 
 /* ------------------------------------------------------------------------- */
+/* Dense backward.
+ * Replaces flash_attn_triton_bwd and its three kernels
+ * (flash_attn_triton/flash_attn_triton.py:661-813, :183-593): given q, k, v,
+ * the forward's o and base-2 lse, and dout = d(loss)/d(o), writes dq, dk, dv
+ * (dtype as q; dk/dv have heads_kv heads: the query heads of a GQA group are
+ * summed inside the kernel).  Addressing modes, causal flag and scale as in
+ * mi_attn_fwd; head_dim 96 or 128.  The workspace holds
+ * Delta = rowsum(o * dout) in fp32.  Four launches on `stream`.
+ */
+typedef struct mi_attn_bwd_args {
+  uint32_t struct_size;
+  int32_t dtype;
+  const void *q, *k, *v, *o, *dout;  /* device                                 */
+  const float *lse;                  /* device, as written by mi_attn_fwd      */
+  void *dq, *dk, *dv;                /* device, fully written for rows < len   */
+  int64_t q_stride_b, q_stride_s, q_stride_h;
+  int64_t k_stride_b, k_stride_s, k_stride_h;
+  int64_t v_stride_b, v_stride_s, v_stride_h;
+  int64_t o_stride_b, o_stride_s, o_stride_h;
+  int64_t dout_stride_b, dout_stride_s, dout_stride_h;
+  int64_t dq_stride_b, dq_stride_s, dq_stride_h;
+  int64_t dk_stride_b, dk_stride_s, dk_stride_h;
+  int64_t dv_stride_b, dv_stride_s, dv_stride_h;
+  int64_t lse_stride_b, lse_stride_s, lse_stride_h;
+  const int32_t *cu_seqlens;         /* device [batch+1] or NULL               */
+  int32_t batch, heads_q, heads_kv;
+  int32_t max_seqlen;
+  int32_t head_dim;                  /* 96 or 128                              */
+  int32_t causal;
+  float scale_log2;                  /* the value the forward pass was given   */
+  void *workspace;                   /* device, mi_attn_bwd_workspace_bytes()  */
+  size_t workspace_bytes;
+} mi_attn_bwd_args;
+
+size_t mi_attn_bwd_workspace_bytes(const mi_attn_bwd_args *args);
+int mi_attn_bwd(const mi_attn_bwd_args *args, void *stream);
+
+/* ------------------------------------------------------------------------- */
 /* Block-sparse forward (always token-causal).
  * Replaces the sparse launcher + kernel of
  * flash_attn_triton/flash_attn_sparse_attn_triton.py:237-326, :47-234, whose
@@ -267,12 +305,13 @@ const char *mi_status_name(int status);
 int mi_attn_fwd_validate(const mi_attn_fwd_args *args);
 int mi_attn_fwd_blocksparse_validate(const mi_attn_sparse_args *args);
 int mi_decode_validate(const mi_decode_args *args);
+int mi_attn_bwd_validate(const mi_attn_bwd_args *args);
 
 /* Average device time per launch, measured with HIP events on `stream` around
  * `iters` back-to-back launches of the given entry point (after `warmup`
  * untimed ones).  Blocks the calling thread; for benchmarking only.
  * kind: 0 = mi_attn_fwd, 1 = mi_attn_fwd_blocksparse, 2 = mi_decode,
- *       3 = mi_decode_splitkv, 4 = mi_decode_merge.
+ *       3 = mi_decode_splitkv, 4 = mi_decode_merge, 5 = mi_attn_bwd.
  * Returns MI_OK and writes milliseconds to *ms_per_launch. */
 int mi_time_launches(int kind, const void *args, void *stream, int warmup,
                      int iters, float *ms_per_launch);

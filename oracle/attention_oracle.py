@@ -14,7 +14,7 @@ triple-loop evaluation of softmax(q.k*scale + mask).v, against
 torch.nn.functional.scaled_dot_product_attention where the mask is expressible,
 and against closed forms (zero queries -> running mean of v, a single key ->
 v itself, one-hot huge queries -> row selection, split invariance of the
-merge).  Parity against the third-party `flash_attn` wheel, which the reference
+merge); the backward formulas against torch.autograd through the forward.  Parity against the third-party `flash_attn` wheel, which the reference
 uses as a second oracle (flash_attn_triton/flash_attn_triton.py:965-975), is
 UNPINNED: that wheel is not installed and is not vendored by the reference.
 """
@@ -103,6 +103,49 @@ def varlen_masked_attention(q, k, v, cu_seq_lens, mask_fn, scale=None, faithful=
             l2 = l2.masked_fill(dead[None], float("-inf"))
             lse[0, s:e] = l2.transpose(0, 1)
     return (o, lse) if return_lse else o
+
+
+def varlen_masked_attention_backward(q, k, v, do, cu_seq_lens, mask_fn, scale=None):
+    """Gradients of varlen_masked_attention(faithful=False) with respect to q, k
+    and v for an upstream gradient `do`, by the closed formulas the reference's
+    backward kernels implement (flash_attn_triton/flash_attn_triton.py:183-593;
+    its test compares them with autograd through the torch path, :1086-1089):
+        P = softmax(S),  dV = P^T dO,  dP = dO V^T,  Delta = rowsum(dO o O),
+        dS = P o (dP - Delta),  dQ = dS K scale,  dK = dS^T Q scale,
+    in float64, the gradients of the query heads sharing a kv-head summed
+    (:687-692,813).  q/do [1,T,Hq,D], k/v [1,T,Hkv,D]; returns float64
+    (dq, dk, dv) of the same shapes.  Pinned against torch.autograd in
+    tests/test_oracle.py."""
+    _, T, H, D = q.shape
+    hkv = k.shape[2]
+    g = H // hkv
+    if scale is None:
+        scale = (1 / D) ** 0.5
+    dq = torch.zeros(1, T, H, D, dtype=torch.float64)
+    dk = torch.zeros(1, T, hkv, D, dtype=torch.float64)
+    dv = torch.zeros(1, T, hkv, D, dtype=torch.float64)
+    for s, e in _lengths(cu_seq_lens):
+        L = e - s
+        if L == 0:
+            continue
+        keep = mask_fn(L)
+        qq, dd = q[0, s:e].double(), do[0, s:e].double()            # [L, H, D]
+        kk = k[0, s:e].double().repeat_interleave(g, dim=1)
+        vv = v[0, s:e].double().repeat_interleave(g, dim=1)
+        sc = torch.einsum("qhd,khd->hqk", qq, kk) * scale
+        sc = sc.masked_fill(~keep[None], float("-inf"))
+        dead = ~keep.any(-1)
+        p = torch.softmax(sc.masked_fill(dead[None, :, None], 0.0), dim=-1).masked_fill(dead[None, :, None], 0.0)
+        o = torch.einsum("hqk,khd->qhd", p, vv)
+        delta = (o * dd).sum(-1).transpose(0, 1)                    # [H, L]
+        dp = torch.einsum("qhd,khd->hqk", dd, vv)
+        ds = p * (dp - delta[:, :, None])
+        dq[0, s:e] = torch.einsum("hqk,khd->qhd", ds, kk) * scale
+        dk_h = torch.einsum("hqk,qhd->khd", ds, qq) * scale          # per q-head
+        dv_h = torch.einsum("hqk,qhd->khd", p, dd)
+        dk[0, s:e] = dk_h.reshape(L, hkv, g, D).sum(2)
+        dv[0, s:e] = dv_h.reshape(L, hkv, g, D).sum(2)
+    return dq, dk, dv
 
 
 def causal_mask(L):

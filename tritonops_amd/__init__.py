@@ -7,6 +7,7 @@ from .ops import (  # noqa: F401
     flash_attention_sparse_decoding,
     flash_attn_sparse_triton,
     flash_attn_triton,
+    flash_attn_triton_bwd,
     flash_attn_triton_fwd,
 )
 from . import masks  # noqa: F401

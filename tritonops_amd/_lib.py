@@ -70,6 +70,21 @@ class AttnSparseArgs(C.Structure):
     ]
 
 
+class AttnBwdArgs(C.Structure):
+    _fields_ = (
+        [("struct_size", _u32), ("dtype", _i32),
+         ("q", _vp), ("k", _vp), ("v", _vp), ("o", _vp), ("dout", _vp), ("lse", _vp),
+         ("dq", _vp), ("dk", _vp), ("dv", _vp)]
+        + [("%s_stride_%s" % (t, d), _i64) for t in ("q", "k", "v", "o", "dout", "dq", "dk", "dv", "lse")
+           for d in ("b", "s", "h")]
+        + [("cu_seqlens", _vp),
+           ("batch", _i32), ("heads_q", _i32), ("heads_kv", _i32),
+           ("max_seqlen", _i32), ("head_dim", _i32), ("causal", _i32),
+           ("scale_log2", _f32),
+           ("workspace", _vp), ("workspace_bytes", _sz)]
+    )
+
+
 class DecodeArgs(C.Structure):
     _fields_ = [
         ("struct_size", _u32), ("dtype", _i32),
@@ -98,6 +113,9 @@ class DecodeArgs(C.Structure):
 EXPORTS = {
     "mi_attn_fwd": (C.c_int, [C.POINTER(AttnFwdArgs), _vp]),
     "mi_attn_fwd_blocksparse": (C.c_int, [C.POINTER(AttnSparseArgs), _vp]),
+    "mi_attn_bwd": (C.c_int, [C.POINTER(AttnBwdArgs), _vp]),
+    "mi_attn_bwd_workspace_bytes": (_sz, [C.POINTER(AttnBwdArgs)]),
+    "mi_attn_bwd_validate": (C.c_int, [C.POINTER(AttnBwdArgs)]),
     "mi_decode_num_splits": (C.c_int, [C.POINTER(DecodeArgs)]),
     "mi_decode_workspace_bytes": (_sz, [C.POINTER(DecodeArgs)]),
     "mi_decode_choose_split_tokens": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int]),

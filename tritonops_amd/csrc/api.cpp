@@ -155,6 +155,75 @@ int mi_attn_fwd_validate(const mi_attn_fwd_args* a) {
   return MI_OK;
 }
 
+int mi_attn_bwd_validate(const mi_attn_bwd_args* a) {
+  if (!a) return fail(MI_ERR_NULL_POINTER, "args is NULL");
+  if (a->struct_size != sizeof(mi_attn_bwd_args))
+    return fail(MI_ERR_STRUCT_SIZE, "mi_attn_bwd_args.struct_size %u != %zu", a->struct_size, sizeof(mi_attn_bwd_args));
+  int rc = check_common(a->dtype, a->head_dim, a->batch, a->heads_q, a->heads_kv, a->max_seqlen, a->scale_log2);
+  if (rc) return rc;
+  if (a->head_dim != 96 && a->head_dim != 128)
+    return fail(MI_ERR_HEAD_DIM, "backward supports head_dim 96 and 128 (got %d)", a->head_dim);
+  if (a->max_seqlen == 0) return MI_OK;
+  const void* ptrs[] = {a->q, a->k, a->v, a->o, a->dout, a->lse, a->dq, a->dk, a->dv};
+  for (const void* x : ptrs)
+    if (!x) return fail(MI_ERR_NULL_POINTER, "q, k, v, o, dout, lse, dq, dk and dv must be non-NULL");
+  const void* al[] = {a->q, a->k, a->v, a->o, a->dout, a->dq, a->dk, a->dv};
+  for (const void* x : al)
+    if (!aligned16(x)) return fail(MI_ERR_ALIGNMENT, "q, k, v, o, dout, dq, dk and dv must be 16-byte aligned");
+  const int64_t st[] = {a->q_stride_s, a->q_stride_h, a->k_stride_s, a->k_stride_h, a->v_stride_s, a->v_stride_h,
+                        a->o_stride_s, a->o_stride_h, a->dout_stride_s, a->dout_stride_h, a->dq_stride_s,
+                        a->dq_stride_h, a->dk_stride_s, a->dk_stride_h, a->dv_stride_s, a->dv_stride_h};
+  for (int64_t x : st)
+    if (!mult8(x)) return fail(MI_ERR_STRIDE, "tensor strides must be multiples of 8 elements (got %lld)", (long long)x);
+  if (!a->cu_seqlens) {
+    const int64_t sb[] = {a->q_stride_b, a->k_stride_b, a->v_stride_b, a->o_stride_b, a->dout_stride_b,
+                          a->dq_stride_b, a->dk_stride_b, a->dv_stride_b};
+    for (int64_t x : sb)
+      if (!mult8(x)) return fail(MI_ERR_STRIDE, "batch strides must be multiples of 8 elements (got %lld)", (long long)x);
+  }
+  if (a->causal != 0 && a->causal != 1) return fail(MI_ERR_SHAPE, "causal must be 0 or 1");
+  const long long wgs = (long long)((a->max_seqlen + 255) / 256) * a->heads_q * a->batch;
+  if (wgs > 0x7fffffffLL || a->heads_q > 65535 || a->batch > 65535)
+    return fail(MI_ERR_SHAPE, "launch grid too large");
+  if (!a->workspace || a->workspace_bytes < mi_attn_bwd_workspace_bytes(a))
+    return fail(MI_ERR_WORKSPACE, "workspace of %zu bytes needed", mi_attn_bwd_workspace_bytes(a));
+  if (!aligned16(a->workspace)) return fail(MI_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
+  return MI_OK;
+}
+
+size_t mi_attn_bwd_workspace_bytes(const mi_attn_bwd_args* a) {
+  if (!a || a->batch <= 0 || a->heads_q <= 0 || a->max_seqlen <= 0) return 0;
+  return (size_t)a->batch * a->heads_q * (size_t)a->max_seqlen * sizeof(float);
+}
+
+int mi_attn_bwd(const mi_attn_bwd_args* a, void* stream) {
+  int rc = mi_attn_bwd_validate(a);
+  if (rc) return rc;
+  if (a->max_seqlen == 0) return MI_OK;
+  mi::BwdParams p;
+  std::memset(&p, 0, sizeof(p));
+  p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o; p.dout = a->dout; p.lse = a->lse;
+  p.delta = static_cast<float*>(a->workspace);
+  p.dq = a->dq; p.dk = a->dk; p.dv = a->dv;
+  p.q_sb = a->q_stride_b; p.q_ss = a->q_stride_s; p.q_sh = a->q_stride_h;
+  p.k_sb = a->k_stride_b; p.k_ss = a->k_stride_s; p.k_sh = a->k_stride_h;
+  p.v_sb = a->v_stride_b; p.v_ss = a->v_stride_s; p.v_sh = a->v_stride_h;
+  p.o_sb = a->o_stride_b; p.o_ss = a->o_stride_s; p.o_sh = a->o_stride_h;
+  p.do_sb = a->dout_stride_b; p.do_ss = a->dout_stride_s; p.do_sh = a->dout_stride_h;
+  p.dq_sb = a->dq_stride_b; p.dq_ss = a->dq_stride_s; p.dq_sh = a->dq_stride_h;
+  p.dk_sb = a->dk_stride_b; p.dk_ss = a->dk_stride_s; p.dk_sh = a->dk_stride_h;
+  p.dv_sb = a->dv_stride_b; p.dv_ss = a->dv_stride_s; p.dv_sh = a->dv_stride_h;
+  p.lse_sb = a->lse_stride_b; p.lse_ss = a->lse_stride_s; p.lse_sh = a->lse_stride_h;
+  p.dl_sh = a->max_seqlen; p.dl_sb = (int64_t)a->heads_q * a->max_seqlen;
+  p.cu = a->cu_seqlens;
+  p.batch = a->batch; p.hq = a->heads_q; p.hkv = a->heads_kv; p.max_seqlen = a->max_seqlen;
+  p.n_rtiles = (a->max_seqlen + 255) / 256;
+  p.causal = a->causal;
+  p.scale = a->scale_log2;
+  p.scale_nat = a->scale_log2 * 0.6931471805599453f;
+  return launch_status(mi::launch_attn_bwd(p, a->dtype, a->head_dim, static_cast<hipStream_t>(stream)), "mi_attn_bwd");
+}
+
 int mi_attn_fwd(const mi_attn_fwd_args* a, void* stream) {
   int rc = mi_attn_fwd_validate(a);
   if (rc) return rc;
@@ -321,13 +390,14 @@ int mi_decode(const mi_decode_args* a, void* stream) {
 
 int mi_time_launches(int kind, const void* args, void* stream, int warmup, int iters, float* ms_per_launch) {
   if (!args || !ms_per_launch) return fail(MI_ERR_NULL_POINTER, "args / ms_per_launch is NULL");
-  if (iters <= 0 || warmup < 0 || kind < 0 || kind > 4) return fail(MI_ERR_SHAPE, "bad kind / warmup / iters");
+  if (iters <= 0 || warmup < 0 || kind < 0 || kind > 5) return fail(MI_ERR_SHAPE, "bad kind / warmup / iters");
   auto once = [&]() -> int {
     switch (kind) {
       case 0: return mi_attn_fwd(static_cast<const mi_attn_fwd_args*>(args), stream);
       case 1: return mi_attn_fwd_blocksparse(static_cast<const mi_attn_sparse_args*>(args), stream);
       case 2: return mi_decode(static_cast<const mi_decode_args*>(args), stream);
       case 3: return mi_decode_splitkv(static_cast<const mi_decode_args*>(args), stream);
+      case 5: return mi_attn_bwd(static_cast<const mi_attn_bwd_args*>(args), stream);
       default: return mi_decode_merge(static_cast<const mi_decode_args*>(args), stream);
     }
   };

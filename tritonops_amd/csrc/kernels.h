@@ -58,11 +58,36 @@ struct DecodeParams {
   int64_t pt_sb;
 };
 
+struct BwdParams {
+  const void *q, *k, *v, *o, *dout;
+  const float* lse;  // base-2 row log-sum-exp of the forward pass
+  float* delta;      // workspace [batch][hq][max_seqlen] fp32
+  void *dq, *dk, *dv;
+  int64_t q_sb, q_ss, q_sh;
+  int64_t k_sb, k_ss, k_sh;
+  int64_t v_sb, v_ss, v_sh;
+  int64_t o_sb, o_ss, o_sh;
+  int64_t do_sb, do_ss, do_sh;
+  int64_t dq_sb, dq_ss, dq_sh;
+  int64_t dk_sb, dk_ss, dk_sh;
+  int64_t dv_sb, dv_ss, dv_sh;
+  int64_t lse_sb, lse_ss, lse_sh;
+  int64_t dl_sb, dl_sh;
+  const int32_t* cu;  // null => batched
+  int32_t batch, hq, hkv, max_seqlen;
+  int32_t n_rtiles;   // ceil(max_seqlen / 256)
+  int32_t causal;
+  float scale;        // log2 domain
+  float scale_nat;    // natural base (= scale * ln 2)
+};
+
 // dtype: 0 bf16, 1 f16.  head_dim in {64, 96, 128}.  Return hipError_t as int.
 int launch_prefill_dense(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);
 int launch_prefill_sparse(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);
 int launch_decode_splitkv(const DecodeParams& p, int dtype, int head_dim, hipStream_t s);
 int launch_decode_merge(const DecodeParams& p, int dtype, int head_dim, hipStream_t s);
+// head_dim in {96, 128}: delta, dq, dk, dv kernels in that order
+int launch_attn_bwd(const BwdParams& p, int dtype, int head_dim, hipStream_t s);
 
 // Query rows per workgroup of the two prefill kernels.
 constexpr int kDenseRows = 256;

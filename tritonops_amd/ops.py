@@ -103,6 +103,53 @@ def _dense_fwd(q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, want_lse=T
     return o, lse
 
 
+def _dense_bwd(q, k, v, o, lse, do, cu_seq_lens, scale_log2, causal, max_seq_len):
+    """q, k, v, o, do as [X, S, H, D] views, lse [X, S, H] (see _fill_qkvo).
+    Returns dq, dk, dv shaped and laid out like q, k, v."""
+    _require_gpu(q, k, v, o, do, lse, cu_seq_lens)
+    lib = _lib.load()
+    q, k, v, o, do = (_inner_contig(t) for t in (q, k, v, o, do))
+    packed = cu_seq_lens is not None
+    X, S, Hq, D = q.shape
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    a = _lib.AttnBwdArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _dtype_tag(q)
+    for name, t in (("q", q), ("k", k), ("v", v), ("o", o), ("dout", do), ("dq", dq), ("dk", dk), ("dv", dv),
+                    ("lse", lse)):
+        setattr(a, name, _ptr(t))
+        setattr(a, name + "_stride_b", 0 if packed else t.stride(0))
+        setattr(a, name + "_stride_s", t.stride(1))
+        setattr(a, name + "_stride_h", t.stride(2))
+    if packed:
+        cu = cu_seq_lens.to(torch.int32)
+        a.cu_seqlens = _ptr(cu)
+        a.batch = cu.numel() - 1
+        a.max_seqlen = min(_max_len(cu, max_seq_len), S)
+        # rows outside every sequence receive no gradient
+        dq.zero_(), dk.zero_(), dv.zero_()
+    else:
+        a.cu_seqlens = None
+        a.batch = X
+        a.max_seqlen = S
+    a.heads_q, a.heads_kv, a.head_dim = Hq, k.shape[2], D
+    a.causal = 1 if causal else 0
+    a.scale_log2 = float(scale_log2)
+    nbytes = lib.mi_attn_bwd_workspace_bytes(C.byref(a))
+    ws = torch.empty(max(nbytes, 16), device=q.device, dtype=torch.uint8)
+    a.workspace, a.workspace_bytes = _ptr(ws), nbytes
+    _lib.check(lib.mi_attn_bwd(C.byref(a), _stream()))
+    return dq, dk, dv
+
+
+def flash_attn_triton_bwd(q, k, v, o, lse, do, cu_seq_lens, sm_scale, *, max_seq_len=None):
+    """Causal var-len GQA backward on packed tensors: contract of
+    flash_attn_triton_bwd in flash_attn_triton/flash_attn_triton.py:661-813
+    (`sm_scale` contains log2(e), `lse` is the base-2 LSE the forward returned).
+    Returns (dq, dk, dv) with the shapes of q, k, v; head_dim 96 or 128."""
+    return _dense_bwd(q, k, v, o, lse, do, cu_seq_lens, sm_scale, True, max_seq_len)
+
+
 def flash_attn_triton_fwd(q, k, v, cu_seq_lens, sm_scale, *, max_seq_len=None):
     """Causal var-len GQA forward on packed tensors.
 
@@ -118,9 +165,8 @@ def flash_attn_triton_fwd(q, k, v, cu_seq_lens, sm_scale, *, max_seq_len=None):
 
 class flash_attn_triton(torch.autograd.Function):
     """`flash_attn_triton.apply(q, k, v, cu_seq_lens) -> o`, the autograd entry
-    of flash_attn_triton/flash_attn_triton.py:816-874.  Forward only: the
-    backward kernels (:183-593) are not part of this library yet and
-    `backward` raises."""
+    of flash_attn_triton/flash_attn_triton.py:816-874 (forward :819-846,
+    backward :848-874).  Backward needs head_dim 96 or 128."""
 
     @staticmethod
     def forward(ctx, q, k, v, cu_seq_lens):
@@ -132,7 +178,9 @@ class flash_attn_triton(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, do):
-        raise NotImplementedError("attention backward is not implemented in tritonops_amd")
+        q, k, v, o, lse, cu_seq_lens = ctx.saved_tensors
+        dq, dk, dv = flash_attn_triton_bwd(q, k, v, o, lse, do, cu_seq_lens, ctx.sm_scale)
+        return dq, dk, dv, None
 
 
 def flash_attention(q, k, v, cu_seq_lens=None, *, causal=True, softmax_scale=None,
