@@ -109,10 +109,27 @@ bwd_kernel(const BwdParams p) {
 
   const int heads_r = MODE == kDQ ? p.hq : p.hkv;
   const int gqa = p.hq / p.hkv;
-  const int bid = blockIdx.x;
-  const int rt = p.n_rtiles - 1 - bid % p.n_rtiles;
-  const int hr = (bid / p.n_rtiles) % heads_r;
-  const int b = bid / (p.n_rtiles * heads_r);
+  // Work item -> (sequence, resident head, resident tile).  Consecutive ids go
+  // round-robin to the 8 XCDs (private L2 each): give every XCD whole
+  // (sequence, head) units so the streamed tensors of a unit stay in one L2,
+  // and walk a unit's tiles from the one that streams most to the one that
+  // streams least (causal: the last q tile for DQ, the first key tile for DK/DV).
+  const int n_units = p.batch * heads_r;
+  int unit, slot;
+  {
+    const int bid = blockIdx.x;
+    if ((n_units & 7) == 0) {
+      const int sl = bid >> 3;
+      unit = (sl / p.n_rtiles) * 8 + (bid & 7);
+      slot = sl % p.n_rtiles;
+    } else {
+      unit = bid / p.n_rtiles;
+      slot = bid % p.n_rtiles;
+    }
+  }
+  const int rt = MODE == kDQ ? p.n_rtiles - 1 - slot : slot;
+  const int hr = unit % heads_r;
+  const int b = unit / heads_r;
 
   int len;
   int64_t start;  // first row of the sequence in packed tensors
@@ -243,13 +260,35 @@ bwd_kernel(const BwdParams p) {
         // DQ: keys past this wave's last query; DK/DV: queries before this wave's first key
         if (MODE == kDQ ? (sblk > r0w + 31) : (sblk + 31 < r0w)) continue;
       }
-      f32x16 S = (f32x16){0};
+      // First products: S (and dP) as independent accumulator chains stepped
+      // alternately, row fragments fetched kPrefetch steps ahead of their MFMA.
+      constexpr int NCHAIN = MODE == kDV ? 1 : 2;
+      constexpr int NSTEP = NCHAIN * G::KSTEPS;
+      constexpr int kPrefetch = 4;
+      f32x16 S = (f32x16){0}, dP = (f32x16){0};
+      {
+        i32x4 f[kPrefetch];
+        auto frag = [&](int st) __attribute__((always_inline)) -> i32x4 {
+          return fr.rows((st % NCHAIN) == 0 ? T0 : T1, sb, st / NCHAIN);
+        };
 #pragma unroll
-      for (int c = 0; c < G::KSTEPS; ++c) S = Elem<T>::mfma(fr.rows(T0, sb, c), Xf[c], S);
-      f32x16 dP = (f32x16){0};
-      if (MODE != kDV) {
+        for (int st = 0; st < kPrefetch; ++st) f[st] = frag(st);
 #pragma unroll
-        for (int c = 0; c < G::KSTEPS; ++c) dP = Elem<T>::mfma(fr.rows(T1, sb, c), Yf[c], dP);
+        for (int st = 0; st < NSTEP; ++st) {
+          if ((st % NCHAIN) == 0)
+            S = Elem<T>::mfma(f[st % kPrefetch], Xf[st / NCHAIN], S);
+          else
+            dP = Elem<T>::mfma(f[st % kPrefetch], Yf[st / NCHAIN], dP);
+          if (st + kPrefetch < NSTEP) f[st % kPrefetch] = frag(st + kPrefetch);
+        }
+        // pin that order (the scheduler otherwise sinks each LDS read next to its MFMA)
+        __builtin_amdgcn_sched_group_barrier(0x100, kPrefetch, 0);
+#pragma unroll
+        for (int st = 0; st < NSTEP - kPrefetch; ++st) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, kPrefetch, 0);
       }
       // register r of this lane is streamed row  sblk + 16*(r/8) + 8*lh + r%8
       float lse_r[16], dl_r[16];
