@@ -114,6 +114,48 @@ def run_dense_causal(steps, warmup):
     }
 
 
+def run_dense_bwd(steps, warmup):
+    """Backward of the headline configuration (dq, dk, dv from q, k, v, o, lse, do)."""
+    import tritonops_amd as ta
+    from tritonops_amd import _lib, ops
+    B, H, S, D = 4, 32, 8192, 128
+    q, k, v, do = (_randn((B, H, S, D), s) for s in (0, 1, 2, 3))
+    qs, ks, vs, ds = (t.transpose(1, 2) for t in (q, k, v, do))      # [B,S,H,D] views
+    sm = D ** -0.5 * ta.LOG2E
+    o, lse = ops._dense_fwd(qs, ks, vs, None, sm, True, None, bhsd=True)
+    steps, warmup = max(4, steps // 4), max(2, warmup // 4)         # a step is ~5x the forward
+    fn = lambda: ops._dense_bwd(qs, ks, vs, o, lse, ds, None, sm, True, None)
+    ms = _time_steps(fn, steps, warmup)
+    dq, dk, dv = fn()
+    a = _lib.AttnBwdArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _lib.MI_DTYPE_BF16
+    for n, t in (("q", qs), ("k", ks), ("v", vs), ("o", o), ("dout", ds), ("dq", dq), ("dk", dk), ("dv", dv),
+                 ("lse", lse)):
+        setattr(a, n, t.data_ptr())
+        setattr(a, n + "_stride_b", t.stride(0))
+        setattr(a, n + "_stride_s", t.stride(1))
+        setattr(a, n + "_stride_h", t.stride(2))
+    a.cu_seqlens = None
+    a.batch, a.heads_q, a.heads_kv, a.max_seqlen, a.head_dim, a.causal = B, H, H, S, D, 1
+    a.scale_log2 = sm
+    nb = _lib.load().mi_attn_bwd_workspace_bytes(C.byref(a))
+    ws = torch.empty(nb, device="cuda", dtype=torch.uint8)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), nb
+    kms = _event_ms(5, a, steps, warmup)
+    flop = 2.5 * 2.0 * B * H * S * (S + 1) * D       # 10*D per unmasked (q, k) pair: S, dP, dV, dQ, dK
+    return {
+        "name": "dense_causal_bwd", "ms_per_step": ms, "kernel_ms": kms,
+        "metric": "attn_bwd_tflops", "unit": "TFLOP/s", "value": flop / (ms * 1e-3) / 1e12,
+        "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "kernel": "bwd_delta_kernel + bwd_kernel<bf16,128,{dq,dk,dv}> (four launches)"},
+        "config": {"workload": "dense causal attention bwd bf16 B=4 H=32 S=8192 D=128: dq, dk, dv from q, k, v, o, lse, do",
+                   "flop_per_step": flop,
+                   "note": "the three kernels execute 14*D FLOP per pair (S three times, dP twice); the figure "
+                           "counts the 10*D of a fused backward"},
+    }
+
+
 def run_decode(steps, warmup):
     import tritonops_amd as ta
     B, Hq, Hkv, L, D = 64, 32, 8, 32768, 128
@@ -282,6 +324,7 @@ WORKLOADS = {
     "gqa_decode": run_decode,
     "block_sparse": run_block_sparse,
     "sparse_decode": run_sparse_decode,
+    "dense_causal_bwd": run_dense_bwd,
 }
 
 
@@ -320,6 +363,22 @@ def cpu_baseline(name):
         nb = float(lens.sum()) * Hkv * 2 * D * 2
         return {"value": nb / t / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
                 "sample": "torch-CPU bf16 decode oracle (flash_attn_decoding.py:339-368) on B=8 of the 64 sequences, median of 3",
+                "seconds": t}
+    if name == "dense_causal_bwd":
+        B, H, S, D = 1, 8, 4096, 128
+        q, k, v, do = (torch.randn((B, H, S, D), generator=g).to(torch.bfloat16) for _ in range(4))
+        ts = []
+        for _ in range(3):
+            qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+            o = orc.causal_attention(qq, kk, vv)
+            t0 = time.perf_counter()
+            o.backward(do)
+            ts.append(time.perf_counter() - t0)
+        t = sorted(ts)[1]
+        flop = 2.5 * 2.0 * B * H * S * (S + 1) * D
+        return {"value": flop / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "sample": "torch-CPU autograd backward through the bf16 causal oracle (tutorial/4.4 math) on B=1 H=8 "
+                          "S=4096 D=128, median of 3; same algorithmic-FLOP formula as the GPU figure",
                 "seconds": t}
     return None
 

@@ -106,7 +106,7 @@ int mi_attn_fwd(const mi_attn_fwd_args *args, void *stream);
  * the forward's o and base-2 lse, and dout = d(loss)/d(o), writes dq, dk, dv
  * (dtype as q; dk/dv have heads_kv heads: the query heads of a GQA group are
  * summed inside the kernel).  Addressing modes, causal flag and scale as in
- * mi_attn_fwd; head_dim 96 or 128.  The workspace holds
+ * mi_attn_fwd.  The workspace holds
  * Delta = rowsum(o * dout) in fp32.  Four launches on `stream`.
  */
 typedef struct mi_attn_bwd_args {
@@ -127,7 +127,7 @@ typedef struct mi_attn_bwd_args {
   const int32_t *cu_seqlens;         /* device [batch+1] or NULL               */
   int32_t batch, heads_q, heads_kv;
   int32_t max_seqlen;
-  int32_t head_dim;                  /* 96 or 128                              */
+  int32_t head_dim;                  /* 64, 96 or 128                          */
   int32_t causal;
   float scale_log2;                  /* the value the forward pass was given   */
   void *workspace;                   /* device, mi_attn_bwd_workspace_bytes()  */

@@ -161,8 +161,6 @@ int mi_attn_bwd_validate(const mi_attn_bwd_args* a) {
     return fail(MI_ERR_STRUCT_SIZE, "mi_attn_bwd_args.struct_size %u != %zu", a->struct_size, sizeof(mi_attn_bwd_args));
   int rc = check_common(a->dtype, a->head_dim, a->batch, a->heads_q, a->heads_kv, a->max_seqlen, a->scale_log2);
   if (rc) return rc;
-  if (a->head_dim != 96 && a->head_dim != 128)
-    return fail(MI_ERR_HEAD_DIM, "backward supports head_dim 96 and 128 (got %d)", a->head_dim);
   if (a->max_seqlen == 0) return MI_OK;
   const void* ptrs[] = {a->q, a->k, a->v, a->o, a->dout, a->lse, a->dq, a->dk, a->dv};
   for (const void* x : ptrs)

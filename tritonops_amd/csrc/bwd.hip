@@ -37,14 +37,14 @@ constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (7 << 4)
 
 enum { kDQ = 0, kDK = 1, kDV = 2 };
 
-// Unpadded 256-byte rows, 16-byte chunks XOR-swizzled per row with a pattern
+// 256-byte rows (head_dim 64 and 96 leave the tail of a row unused), 16-byte
+// chunks XOR-swizzled per row with a pattern
 // that is free of bank conflicts for BOTH access patterns: a row-fragment read
 // takes one chunk from 16 rows whose low four row bits are all different, a
 // transposing read takes four consecutive chunks from four consecutive rows.
 template <int D>
 struct UniFrags {
   using G = RowGeom<D>;
-  static_assert(G::DP == 128, "backward supports head_dim 96 and 128");
   static constexpr int ROWB = 256;
   static constexpr int SLOTS = 16;
   static __device__ __forceinline__ int swz(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
@@ -231,7 +231,7 @@ bwd_kernel(const BwdParams p) {
       const int r = RPI * inst + drow;
       const int c = dslot ^ F::swz(r);
       const int64_t rr = min(s0 + r, len - 1);  // rows past the end re-read the last row (masked later)
-      if (D != 96 || c < G::NCH) {
+      if (G::NCH == 16 || c < G::NCH) {
         dma16(t0 + rr * pitch0 + c * 16, base + inst * 1024);
         dma16(t1 + rr * pitch1 + c * 16, base + TILEB + inst * 1024);
       }
@@ -471,9 +471,11 @@ int launch_all(const BwdParams& p, hipStream_t s) {
 
 int launch_attn_bwd(const BwdParams& p, int dtype, int head_dim, hipStream_t s) {
   if (dtype == 0) {
+    if (head_dim == 64) return launch_all<__bf16, 64>(p, s);
     if (head_dim == 96) return launch_all<__bf16, 96>(p, s);
     if (head_dim == 128) return launch_all<__bf16, 128>(p, s);
   } else {
+    if (head_dim == 64) return launch_all<_Float16, 64>(p, s);
     if (head_dim == 96) return launch_all<_Float16, 96>(p, s);
     if (head_dim == 128) return launch_all<_Float16, 128>(p, s);
   }

@@ -86,7 +86,7 @@ int launch_prefill_dense(const PrefillParams& p, int dtype, int head_dim, hipStr
 int launch_prefill_sparse(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);
 int launch_decode_splitkv(const DecodeParams& p, int dtype, int head_dim, hipStream_t s);
 int launch_decode_merge(const DecodeParams& p, int dtype, int head_dim, hipStream_t s);
-// head_dim in {96, 128}: delta, dq, dk, dv kernels in that order
+// delta, dq, dk, dv kernels in that order
 int launch_attn_bwd(const BwdParams& p, int dtype, int head_dim, hipStream_t s);
 
 // Query rows per workgroup of the two prefill kernels.

@@ -146,7 +146,7 @@ def flash_attn_triton_bwd(q, k, v, o, lse, do, cu_seq_lens, sm_scale, *, max_seq
     """Causal var-len GQA backward on packed tensors: contract of
     flash_attn_triton_bwd in flash_attn_triton/flash_attn_triton.py:661-813
     (`sm_scale` contains log2(e), `lse` is the base-2 LSE the forward returned).
-    Returns (dq, dk, dv) with the shapes of q, k, v; head_dim 96 or 128."""
+    Returns (dq, dk, dv) with the shapes of q, k, v."""
     return _dense_bwd(q, k, v, o, lse, do, cu_seq_lens, sm_scale, True, max_seq_len)
 
 
@@ -166,7 +166,7 @@ def flash_attn_triton_fwd(q, k, v, cu_seq_lens, sm_scale, *, max_seq_len=None):
 class flash_attn_triton(torch.autograd.Function):
     """`flash_attn_triton.apply(q, k, v, cu_seq_lens) -> o`, the autograd entry
     of flash_attn_triton/flash_attn_triton.py:816-874 (forward :819-846,
-    backward :848-874).  Backward needs head_dim 96 or 128."""
+    backward :848-874)."""
 
     @staticmethod
     def forward(ctx, q, k, v, cu_seq_lens):
