@@ -260,36 +260,6 @@ bwd_kernel(const BwdParams p) {
         // DQ: keys past this wave's last query; DK/DV: queries before this wave's first key
         if (MODE == kDQ ? (sblk > r0w + 31) : (sblk + 31 < r0w)) continue;
       }
-      // First products: S (and dP) as independent accumulator chains stepped
-      // alternately, row fragments fetched kPrefetch steps ahead of their MFMA.
-      constexpr int NCHAIN = MODE == kDV ? 1 : 2;
-      constexpr int NSTEP = NCHAIN * G::KSTEPS;
-      constexpr int kPrefetch = 4;
-      f32x16 S = (f32x16){0}, dP = (f32x16){0};
-      {
-        i32x4 f[kPrefetch];
-        auto frag = [&](int st) __attribute__((always_inline)) -> i32x4 {
-          return fr.rows((st % NCHAIN) == 0 ? T0 : T1, sb, st / NCHAIN);
-        };
-#pragma unroll
-        for (int st = 0; st < kPrefetch; ++st) f[st] = frag(st);
-#pragma unroll
-        for (int st = 0; st < NSTEP; ++st) {
-          if ((st % NCHAIN) == 0)
-            S = Elem<T>::mfma(f[st % kPrefetch], Xf[st / NCHAIN], S);
-          else
-            dP = Elem<T>::mfma(f[st % kPrefetch], Yf[st / NCHAIN], dP);
-          if (st + kPrefetch < NSTEP) f[st % kPrefetch] = frag(st + kPrefetch);
-        }
-        // pin that order (the scheduler otherwise sinks each LDS read next to its MFMA)
-        __builtin_amdgcn_sched_group_barrier(0x100, kPrefetch, 0);
-#pragma unroll
-        for (int st = 0; st < NSTEP - kPrefetch; ++st) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, kPrefetch, 0);
-      }
       // register r of this lane is streamed row  sblk + 16*(r/8) + 8*lh + r%8
       float lse_r[16], dl_r[16];
       if (ROWVEC) {
@@ -310,37 +280,93 @@ bwd_kernel(const BwdParams p) {
             }
           }
       }
+      // The block as one pinned instruction stream (sched_barrier(0) after every
+      // slice): the S chain; the dP chain with the exponentials of S behind its
+      // MFMAs; the first half of dS; the last product with the second half of
+      // dS behind its first MFMAs.  Row fragments are read four steps ahead,
+      // transposed fragments two.
+      constexpr bool TWO = MODE != kDV;
+      constexpr int NSTEP = (TWO ? 2 : 1) * G::KSTEPS;
+      constexpr int kPrefetch = 4;
+      constexpr uint32_t TT = MODE == kDV ? T1 : T0;  // tile whose transpose is the A operand
+      f32x16 S = (f32x16){0}, dP = (f32x16){0};
+      i32x4 f[kPrefetch];
+      auto frag = [&](int st) __attribute__((always_inline)) -> i32x4 {
+        return st < G::KSTEPS ? fr.rows(T0, sb, st) : fr.rows(T1, sb, st - G::KSTEPS);
+      };
+      auto prob = [&](int r) __attribute__((always_inline)) {   // S[r] <- P[r]
+        S[r] = fast_exp2(fmaf(S[r], scale, -(ROWVEC ? lse_r[r] : lse_l)));
+      };
+      auto dsv = [&](int r) __attribute__((always_inline)) -> float {
+        return MODE == kDV ? S[r] : S[r] * (dP[r] - (ROWVEC ? dl_r[r] : delta_l));
+      };
+#pragma unroll
+      for (int st = 0; st < kPrefetch; ++st) f[st] = frag(st);
+#pragma unroll
+      for (int st = 0; st < G::KSTEPS; ++st) {
+        S = Elem<T>::mfma(f[st % kPrefetch], Xf[st], S);
+        if (st + kPrefetch < NSTEP) f[st % kPrefetch] = frag(st + kPrefetch);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // rare: rows / columns that do not exist or lie above the diagonal give P = 0
       bool need_mask = sblk + 32 > len;
       if (MODE != kDQ) need_mask = need_mask || r0w + 32 > len;
       if (causal) need_mask = need_mask || (MODE == kDQ ? (sblk + 31 > r0w) : (sblk < r0w + 31));
-      uint32_t W[8];
+      if (need_mask) {
 #pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        float w2[2];
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-          const int rr = r + e;
-          const int srow = sblk + 16 * (rr >> 3) + 8 * fr.lh + (rr & 7);
-          const float pr = fast_exp2(fmaf(S[rr], scale, -(ROWVEC ? lse_r[rr] : lse_l)));
-          float val = MODE == kDV ? pr : pr * (dP[rr] - (ROWVEC ? dl_r[rr] : delta_l));
-          if (need_mask) {
-            bool ok;
-            if (MODE == kDQ)
-              ok = srow < len && (!causal || srow <= rrow);
-            else
-              ok = srow < len && rrow < len && (!causal || rrow <= srow);
-            val = ok ? val : 0.f;
-          }
-          w2[e] = val;
+        for (int r = 0; r < 16; ++r) {
+          const int srow = sblk + 16 * (r >> 3) + 8 * fr.lh + (r & 7);
+          bool ok;
+          if (MODE == kDQ)
+            ok = srow < len && (!causal || srow <= rrow);
+          else
+            ok = srow < len && rrow < len && (!causal || rrow <= srow);
+          S[r] = ok ? S[r] : -INFINITY;
         }
-        W[r >> 1] = Elem<T>::pack2(w2[0], w2[1]);
       }
-      constexpr uint32_t TT = MODE == kDV ? T1 : T0;  // tile whose transpose is the A operand
+      i32x4 tf[2];
+      uint32_t W[8];
+      if (TWO) {
 #pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
+        for (int c = 0; c < G::KSTEPS; ++c) {
+          const int st = G::KSTEPS + c;
+          dP = Elem<T>::mfma(f[st % kPrefetch], Yf[c], dP);
+          if (st + kPrefetch < NSTEP) f[st % kPrefetch] = frag(st + kPrefetch);
+          if (c >= G::KSTEPS - 2) tf[c - (G::KSTEPS - 2)] = fr.tr(TT, 2 * sb, c - (G::KSTEPS - 2));
+          // 16 exponentials spread over the KSTEPS slices
+#pragma unroll
+          for (int r = 16 * c / G::KSTEPS; r < 16 * (c + 1) / G::KSTEPS; ++r) prob(r);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+        tf[0] = fr.tr(TT, 2 * sb, 0);
+        tf[1] = fr.tr(TT, 2 * sb, 1);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) prob(r);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) W[i] = Elem<T>::pack2(dsv(2 * i), dsv(2 * i + 1));
+      __builtin_amdgcn_sched_barrier(0);
+      // last product: 2*NDB MFMAs, fragment (kk, db) = step kk*NDB + db
+      constexpr int NACC = 2 * G::NDB;
+#pragma unroll
+      for (int i = 0; i < NACC; ++i) {
+        const int kk = i / G::NDB, db = i % G::NDB;
         const i32x4 wf = {(int)W[4 * kk], (int)W[4 * kk + 1], (int)W[4 * kk + 2], (int)W[4 * kk + 3]};
+        acc[db] = Elem<T>::mfma(tf[i & 1], wf, acc[db]);
+        if (i + 2 < NACC) tf[i & 1] = fr.tr(TT, 2 * sb + (i + 2) / G::NDB, (i + 2) % G::NDB);
+        if (i < G::NDB) {
+          // second half of dS (8 values) spread over the first NDB slices
 #pragma unroll
-        for (int db = 0; db < G::NDB; ++db) acc[db] = Elem<T>::mfma(fr.tr(TT, 2 * sb + kk, db), wf, acc[db]);
+          for (int q = 4 * i / G::NDB; q < 4 * (i + 1) / G::NDB; ++q) {
+            if (!TWO) {
+              prob(8 + 2 * q);
+              prob(9 + 2 * q);
+            }
+            W[4 + q] = Elem<T>::pack2(dsv(8 + 2 * q), dsv(9 + 2 * q));
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   };

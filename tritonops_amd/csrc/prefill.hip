@@ -1,12 +1,14 @@
 // Prefill (many-query) attention forward for gfx950: dense causal / non-causal
 // and block-sparse, packed var-len or batched, GQA.
 //
-// Work decomposition: one workgroup = NW wavefronts = 32*NW consecutive query
-// rows of one (sequence, q-head); KV is walked in tiles of 64 keys that the
-// whole workgroup brings into LDS with direct-to-LDS loads
-// (global_load_lds_dwordx4: no staging registers, no ds_write), double
-// buffered, one barrier per tile; each wavefront then runs compute_tile() on
-// its own 32 rows.
+// Work decomposition: one work item = NW wavefronts x 32 consecutive query
+// rows of one (sequence, q-head); KV is walked in tiles that the whole
+// workgroup brings into an LDS ring with direct-to-LDS loads
+// (global_load_lds_dwordx4: no staging registers, no ds_write), one barrier
+// per tile.  Block-sparse: 32-key tiles, two stages, one launch per item, each
+// wavefront runs compute_tile() on its 32 rows.  Dense: 64-key tiles, four
+// stages, a persistent grid that walks the items, and a software pipeline over
+// half tiles inside each wavefront (see the dense branch of prefill_item).
 //
 // Replaces flash_attn_fwd_kernel of flash_attn_triton/flash_attn_triton.py
 // :52-180 (dense) and flash_attn_triton/flash_attn_sparse_attn_triton.py
@@ -22,9 +24,6 @@
 
 namespace mi {
 namespace {
-
-typedef __attribute__((address_space(3))) void lds_void;
-typedef __attribute__((address_space(1))) const void glb_void;
 
 template <int V>
 using ic = std::integral_constant<int, V>;
