@@ -252,6 +252,9 @@ bwd_kernel(const BwdParams p) {
     constexpr int ST = decltype(stage_c)::value;
     constexpr uint32_t T0 = ST * STAGEB, T1 = ST * STAGEB + TILEB, LV = ST * STAGEB + 2 * TILEB;
     const int s0 = (j0 + u % nj) * TN;
+    constexpr int kPrefetch = 4;
+    i32x4 f[kPrefetch];   // row fragments of the first product, read ahead
+    bool f_ready = false; // block 0 has already fetched the first fragments of block 1
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
       const int sblk = s0 + 32 * sb;
@@ -287,10 +290,8 @@ bwd_kernel(const BwdParams p) {
       // transposed fragments two.
       constexpr bool TWO = MODE != kDV;
       constexpr int NSTEP = (TWO ? 2 : 1) * G::KSTEPS;
-      constexpr int kPrefetch = 4;
       constexpr uint32_t TT = MODE == kDV ? T1 : T0;  // tile whose transpose is the A operand
       f32x16 S = (f32x16){0}, dP = (f32x16){0};
-      i32x4 f[kPrefetch];
       auto frag = [&](int st) __attribute__((always_inline)) -> i32x4 {
         return st < G::KSTEPS ? fr.rows(T0, sb, st) : fr.rows(T1, sb, st - G::KSTEPS);
       };
@@ -300,8 +301,10 @@ bwd_kernel(const BwdParams p) {
       auto dsv = [&](int r) __attribute__((always_inline)) -> float {
         return MODE == kDV ? S[r] : S[r] * (dP[r] - (ROWVEC ? dl_r[r] : delta_l));
       };
+      if (!f_ready) {
 #pragma unroll
-      for (int st = 0; st < kPrefetch; ++st) f[st] = frag(st);
+        for (int st = 0; st < kPrefetch; ++st) f[st] = frag(st);
+      }
 #pragma unroll
       for (int st = 0; st < G::KSTEPS; ++st) {
         S = Elem<T>::mfma(f[st % kPrefetch], Xf[st], S);
@@ -355,6 +358,8 @@ bwd_kernel(const BwdParams p) {
         const i32x4 wf = {(int)W[4 * kk], (int)W[4 * kk + 1], (int)W[4 * kk + 2], (int)W[4 * kk + 3]};
         acc[db] = Elem<T>::mfma(tf[i & 1], wf, acc[db]);
         if (i + 2 < NACC) tf[i & 1] = fr.tr(TT, 2 * sb + (i + 2) / G::NDB, (i + 2) % G::NDB);
+        // the ring is idle now: fetch the first fragments of the tile's second block
+        if (sb == 0 && i >= NACC - kPrefetch) f[i - (NACC - kPrefetch)] = fr.rows(T0, 1, i - (NACC - kPrefetch));
         if (i < G::NDB) {
           // second half of dS (8 values) spread over the first NDB slices
 #pragma unroll
@@ -368,6 +373,7 @@ bwd_kernel(const BwdParams p) {
         }
         __builtin_amdgcn_sched_barrier(0);
       }
+      f_ready = sb == 0;
     }
   };
 
