@@ -319,12 +319,52 @@ def run_sparse_decode(steps, warmup):
     }
 
 
+def run_rmsnorm(steps, warmup):
+    """RMSNorm forward + backward over [32768, 4096] bf16 activations, fp32 weight."""
+    import tritonops_amd as ta
+    from tritonops_amd import _lib
+    T, D, eps = 32768, 4096, 1e-6
+    x, dy = _randn((T, D), 0), _randn((T, D), 1)
+    w = torch.ones(D, device="cuda", dtype=torch.float32)
+
+    def fn():
+        y, rs = ta.rmsnorm_fwd(x, w, eps)
+        return ta.rmsnorm_bwd(dy, x, w, rs, eps)
+    ms = _time_steps(fn, steps, warmup)
+    y, rs = ta.rmsnorm_fwd(x, w, eps)
+    dx, dw = ta.rmsnorm_bwd(dy, x, w, rs, eps)
+    a = _lib.RmsNormArgs()
+    a.struct_size = C.sizeof(a)
+    a.x_dtype, a.w_dtype, a.dim, a.rows = _lib.MI_DTYPE_BF16, _lib.MI_DTYPE_F32, D, T
+    a.x, a.w, a.y, a.rsqrt = x.data_ptr(), w.data_ptr(), y.data_ptr(), rs.data_ptr()
+    a.dy, a.dx, a.dw = dy.data_ptr(), dx.data_ptr(), dw.data_ptr()
+    a.x_stride = a.y_stride = a.dy_stride = a.dx_stride = D
+    a.eps = eps
+    nb = _lib.load().mi_rmsnorm_bwd_workspace_bytes(C.byref(a))
+    ws = torch.empty(nb, device="cuda", dtype=torch.uint8)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), nb
+    k_fwd = _event_ms(6, a, steps, warmup)
+    k_bwd = _event_ms(7, a, steps, warmup)
+    b_fwd = 2.0 * T * D * 2 + T * 4                 # x read, y written, rsqrt written
+    b_bwd = 3.0 * T * D * 2 + T * 4                 # x, dy read, dx written, rsqrt read
+    return {
+        "name": "rmsnorm", "ms_per_step": ms, "kernel_ms": k_fwd + k_bwd,
+        "metric": "rmsnorm_fwd_bwd_hbm_gbs", "unit": "GB/s", "value": (b_fwd + b_bwd) / (ms * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "achieved": (b_fwd + b_bwd) / ((k_fwd + k_bwd) * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "kernel": "rms_fwd_vec_kernel + rms_bwd_vec_kernel + rms_dw_reduce_kernel"},
+        "config": {"workload": "RMSNorm fwd + bwd, x [32768, 4096] bf16, weight fp32, eps 1e-6",
+                   "bytes_per_step": b_fwd + b_bwd, "fwd_kernel_ms": k_fwd, "bwd_kernel_ms": k_bwd,
+                   "fwd_gbs": b_fwd / (k_fwd * 1e-3) / 1e9, "bwd_gbs": b_bwd / (k_bwd * 1e-3) / 1e9},
+    }
+
+
 WORKLOADS = {
     "dense_causal": run_dense_causal,
     "gqa_decode": run_decode,
     "block_sparse": run_block_sparse,
     "sparse_decode": run_sparse_decode,
     "dense_causal_bwd": run_dense_bwd,
+    "rmsnorm": run_rmsnorm,
 }
 
 
@@ -379,6 +419,22 @@ def cpu_baseline(name):
         return {"value": flop / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
                 "sample": "torch-CPU autograd backward through the bf16 causal oracle (tutorial/4.4 math) on B=1 H=8 "
                           "S=4096 D=128, median of 3; same algorithmic-FLOP formula as the GPU figure",
+                "seconds": t}
+    if name == "rmsnorm":
+        from oracle import rms_oracle as rorc
+        T, D, eps = 4096, 4096, 1e-6
+        x, dy = (torch.randn((T, D), generator=g).to(torch.bfloat16) for _ in range(2))
+        w = torch.ones(D)
+
+        def fn():
+            rorc.rms_norm(x.float(), w, eps).to(torch.bfloat16)
+            rorc.rms_norm_backward(dy.float(), x.float(), w, eps)
+        t = med(fn)
+        nbytes = 5.0 * T * D * 2 + 2 * T * 4
+        return {"value": nbytes / t / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+                "sample": "torch-CPU RMSNorm forward (fp32 math, bf16 result) + float64 backward formulas of the oracle "
+                          "(common/rms.py math) on [4096, 4096] bf16 (1/8 of the rows), median of 3; same "
+                          "algorithmic-byte formula as the GPU figure",
                 "seconds": t}
     return None
 

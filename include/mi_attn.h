@@ -43,7 +43,8 @@ extern "C" {
 
 typedef enum mi_dtype {
   MI_DTYPE_BF16 = 0,
-  MI_DTYPE_F16 = 1
+  MI_DTYPE_F16 = 1,
+  MI_DTYPE_F32 = 2            /* mi_rmsnorm_* only                             */
 } mi_dtype;
 
 typedef enum mi_status {
@@ -295,6 +296,41 @@ int mi_decode_merge(const mi_decode_args *args, void *stream);
 int mi_decode(const mi_decode_args *args, void *stream);
 
 /* ------------------------------------------------------------------------- */
+/* RMSNorm forward / backward over rows of `dim` elements.
+ * Replaces RMSNormTritonFunction.forward / .backward and their kernels
+ * (common/rms.py:221-355, :8-218):
+ *   rsqrt[t] = 1 / sqrt(eps + mean_d x[t,d]^2)         fp32, saved for backward
+ *   y[t,d]   = x[t,d] * rsqrt[t] * w[d]
+ *   dx[t,d]  = dy[t,d] w[d] rsqrt[t] - x[t,d] rsqrt[t]^3 (sum_d dy w x) / dim
+ *   dw[d]    = sum_t dy[t,d] x[t,d] rsqrt[t]
+ * x, y, dy, dx share one dtype (MI_DTYPE_BF16, MI_DTYPE_F16 or MI_DTYPE_F32),
+ * rows contiguous with the given row strides (elements); w and dw have the
+ * same dtype as x or are fp32.  Any dim >= 1 (the reference's test uses 255).
+ * The backward needs mi_rmsnorm_bwd_workspace_bytes() of device workspace for
+ * the partial dw rows (no atomics: results are deterministic).
+ */
+typedef struct mi_rmsnorm_args {
+  uint32_t struct_size;
+  int32_t x_dtype;               /* of x, y, dy, dx                            */
+  int32_t w_dtype;               /* of w, dw: x_dtype or MI_DTYPE_F32          */
+  int32_t dim;
+  int64_t rows;
+  const void *x, *w;             /* device                                     */
+  void *y;                       /* forward output                             */
+  float *rsqrt;                  /* [rows]: forward output, backward input     */
+  const void *dy;                /* backward input                             */
+  void *dx, *dw;                 /* backward outputs                           */
+  int64_t x_stride, y_stride, dy_stride, dx_stride;  /* row strides            */
+  float eps;
+  void *workspace;               /* backward only                              */
+  size_t workspace_bytes;
+} mi_rmsnorm_args;
+
+int mi_rmsnorm_fwd(const mi_rmsnorm_args *args, void *stream);
+size_t mi_rmsnorm_bwd_workspace_bytes(const mi_rmsnorm_args *args);
+int mi_rmsnorm_bwd(const mi_rmsnorm_args *args, void *stream);
+
+/* ------------------------------------------------------------------------- */
 /* Introspection (host only). */
 int mi_abi_version(void);
 /* Message of the last failing call on this thread ("" if none). */
@@ -311,7 +347,8 @@ int mi_attn_bwd_validate(const mi_attn_bwd_args *args);
  * `iters` back-to-back launches of the given entry point (after `warmup`
  * untimed ones).  Blocks the calling thread; for benchmarking only.
  * kind: 0 = mi_attn_fwd, 1 = mi_attn_fwd_blocksparse, 2 = mi_decode,
- *       3 = mi_decode_splitkv, 4 = mi_decode_merge, 5 = mi_attn_bwd.
+ *       3 = mi_decode_splitkv, 4 = mi_decode_merge, 5 = mi_attn_bwd,
+ *       6 = mi_rmsnorm_fwd, 7 = mi_rmsnorm_bwd.
  * Returns MI_OK and writes milliseconds to *ms_per_launch. */
 int mi_time_launches(int kind, const void *args, void *stream, int warmup,
                      int iters, float *ms_per_launch);

@@ -32,16 +32,20 @@ def test_every_declared_symbol_is_exported(lib):
 
 def test_struct_layout_matches_the_c_compiler(tmp_path):
     src = tmp_path / "sz.c"
-    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "mi_attn.h"\nint main(){printf("%zu %zu %zu %zu %zu %zu\\n",'
+    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "mi_attn.h"\nint main(){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\\n",'
                    "sizeof(mi_attn_fwd_args),sizeof(mi_attn_sparse_args),sizeof(mi_decode_args),"
                    "offsetof(mi_attn_fwd_args,scale_log2),offsetof(mi_attn_sparse_args,scale_log2),"
-                   "offsetof(mi_decode_args,page_table));return 0;}\n")
+                   "offsetof(mi_decode_args,page_table),"
+                   "sizeof(mi_attn_bwd_args),offsetof(mi_attn_bwd_args,workspace),"
+                   "sizeof(mi_rmsnorm_args),offsetof(mi_rmsnorm_args,eps));return 0;}\n")
     exe = tmp_path / "sz"
     subprocess.check_call(["gcc", "-std=c99", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
     got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
     want = [C.sizeof(_lib.AttnFwdArgs), C.sizeof(_lib.AttnSparseArgs), C.sizeof(_lib.DecodeArgs),
             _lib.AttnFwdArgs.scale_log2.offset, _lib.AttnSparseArgs.scale_log2.offset,
-            _lib.DecodeArgs.page_table.offset]
+            _lib.DecodeArgs.page_table.offset,
+            C.sizeof(_lib.AttnBwdArgs), _lib.AttnBwdArgs.workspace.offset,
+            C.sizeof(_lib.RmsNormArgs), _lib.RmsNormArgs.eps.offset]
     assert got == want
 
 
@@ -204,6 +208,46 @@ def test_split_heuristic(lib):
     assert f(64, 8, 32768, 256) <= 4096
     assert f(1, 1, 1 << 20, 256) == 256          # one sequence: as many chunks as allowed
     assert f(4096, 8, 4096, 256) == 4096         # plenty of sequences: one chunk each
+
+
+def test_backward_and_rmsnorm_validation(lib):
+    a = _lib.AttnBwdArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype, a.batch, a.heads_q, a.heads_kv, a.max_seqlen, a.head_dim, a.causal = 0, 1, 4, 2, 128, 128, 1
+    a.scale_log2 = 0.1
+    for n in ("q", "k", "v", "o", "dout", "lse", "dq", "dk", "dv"):
+        setattr(a, n, 0x1000)
+        for d in ("b", "s", "h"):
+            setattr(a, "%s_stride_%s" % (n, d), 1024)
+    assert lib.mi_attn_bwd_workspace_bytes(C.byref(a)) == 1 * 4 * 128 * 4
+    assert lib.mi_status_name(lib.mi_attn_bwd_validate(C.byref(a))).decode() == "MI_ERR_WORKSPACE"
+    a.workspace, a.workspace_bytes = 0x2000, 4096
+    assert lib.mi_attn_bwd_validate(C.byref(a)) == 0
+    a.dk = None
+    assert lib.mi_status_name(lib.mi_attn_bwd_validate(C.byref(a))).decode() == "MI_ERR_NULL_POINTER"
+    a.dk, a.heads_kv = 0x1000, 3
+    assert lib.mi_status_name(lib.mi_attn_bwd_validate(C.byref(a))).decode() == "MI_ERR_GQA"
+    a.heads_kv, a.struct_size = 2, 8
+    assert lib.mi_attn_bwd(C.byref(a), None) == -2
+
+    r = _lib.RmsNormArgs()
+    r.struct_size = C.sizeof(r)
+    r.x_dtype, r.w_dtype, r.dim, r.rows = 0, 2, 255, 10
+    r.x = r.w = r.y = r.rsqrt = 0x1000
+    r.x_stride = r.y_stride = 255
+    r.eps = 1e-6
+    # a launch would follow a clean validation, so only the failing cases are called here
+    r.w_dtype = 1
+    assert lib.mi_status_name(lib.mi_rmsnorm_fwd(C.byref(r), None)).decode() == "MI_ERR_DTYPE"
+    r.w_dtype, r.x_stride = 2, 100
+    assert lib.mi_status_name(lib.mi_rmsnorm_fwd(C.byref(r), None)).decode() == "MI_ERR_STRIDE"
+    r.x_stride, r.dim = 255, 0
+    assert lib.mi_status_name(lib.mi_rmsnorm_fwd(C.byref(r), None)).decode() == "MI_ERR_SHAPE"
+    r.dim = 255
+    assert lib.mi_status_name(lib.mi_rmsnorm_bwd(C.byref(r), None)).decode() == "MI_ERR_NULL_POINTER"
+    assert lib.mi_rmsnorm_bwd_workspace_bytes(C.byref(r)) == (12 + 32) * 255 * 4  # 10 rows -> 12 partial rows + 32 stage rows
+    r.rows = 0
+    assert lib.mi_rmsnorm_fwd(C.byref(r), None) == 0 and lib.mi_rmsnorm_bwd(C.byref(r), None) == 0
 
 
 def test_split_blocks_heuristic(lib):

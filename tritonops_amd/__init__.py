@@ -10,4 +10,5 @@ from .ops import (  # noqa: F401
     flash_attn_triton_bwd,
     flash_attn_triton_fwd,
 )
+from .rms import RMSNormTriton, RMSNormTritonFunction, rmsnorm_bwd, rmsnorm_fwd  # noqa: F401
 from . import masks  # noqa: F401

@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_HERE, "libmi_attn.so")
 MI_ATTN_ABI_VERSION = 2
 MI_KV_BATCHED, MI_KV_PACKED, MI_KV_PAGED = 0, 1, 2
 MI_ATTN_BLOCK = 64
+MI_DTYPE_F32 = 2
 MI_DTYPE_BF16 = 0
 MI_DTYPE_F16 = 1
 
@@ -85,6 +86,17 @@ class AttnBwdArgs(C.Structure):
     )
 
 
+class RmsNormArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", _u32), ("x_dtype", _i32), ("w_dtype", _i32), ("dim", _i32),
+        ("rows", _i64),
+        ("x", _vp), ("w", _vp), ("y", _vp), ("rsqrt", _vp), ("dy", _vp), ("dx", _vp), ("dw", _vp),
+        ("x_stride", _i64), ("y_stride", _i64), ("dy_stride", _i64), ("dx_stride", _i64),
+        ("eps", _f32),
+        ("workspace", _vp), ("workspace_bytes", _sz),
+    ]
+
+
 class DecodeArgs(C.Structure):
     _fields_ = [
         ("struct_size", _u32), ("dtype", _i32),
@@ -116,6 +128,9 @@ EXPORTS = {
     "mi_attn_bwd": (C.c_int, [C.POINTER(AttnBwdArgs), _vp]),
     "mi_attn_bwd_workspace_bytes": (_sz, [C.POINTER(AttnBwdArgs)]),
     "mi_attn_bwd_validate": (C.c_int, [C.POINTER(AttnBwdArgs)]),
+    "mi_rmsnorm_fwd": (C.c_int, [C.POINTER(RmsNormArgs), _vp]),
+    "mi_rmsnorm_bwd": (C.c_int, [C.POINTER(RmsNormArgs), _vp]),
+    "mi_rmsnorm_bwd_workspace_bytes": (_sz, [C.POINTER(RmsNormArgs)]),
     "mi_decode_num_splits": (C.c_int, [C.POINTER(DecodeArgs)]),
     "mi_decode_workspace_bytes": (_sz, [C.POINTER(DecodeArgs)]),
     "mi_decode_choose_split_tokens": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int]),

@@ -155,6 +155,80 @@ int mi_attn_fwd_validate(const mi_attn_fwd_args* a) {
   return MI_OK;
 }
 
+static int rms_elem_bytes(int dt) { return dt == MI_DTYPE_F32 ? 4 : 2; }
+
+static int rms_validate(const mi_rmsnorm_args* a, bool backward) {
+  if (!a) return fail(MI_ERR_NULL_POINTER, "args is NULL");
+  if (a->struct_size != sizeof(mi_rmsnorm_args))
+    return fail(MI_ERR_STRUCT_SIZE, "mi_rmsnorm_args.struct_size %u != %zu", a->struct_size, sizeof(mi_rmsnorm_args));
+  if (a->x_dtype != MI_DTYPE_BF16 && a->x_dtype != MI_DTYPE_F16 && a->x_dtype != MI_DTYPE_F32)
+    return fail(MI_ERR_DTYPE, "x_dtype %d is not bf16 / f16 / f32", a->x_dtype);
+  if (a->w_dtype != a->x_dtype && a->w_dtype != MI_DTYPE_F32)
+    return fail(MI_ERR_DTYPE, "w_dtype %d must equal x_dtype or be f32", a->w_dtype);
+  if (a->dim <= 0 || a->rows < 0) return fail(MI_ERR_SHAPE, "dim %d must be positive, rows %lld non-negative", a->dim, (long long)a->rows);
+  if (!(a->eps >= 0.f) || !std::isfinite(a->eps)) return fail(MI_ERR_SCALE, "eps must be finite and >= 0");
+  if (a->rows == 0) return MI_OK;
+  if (a->rows > 0x7fffffffLL * 4) return fail(MI_ERR_SHAPE, "too many rows");
+  if (!a->x || !a->w || !a->rsqrt) return fail(MI_ERR_NULL_POINTER, "x, w and rsqrt must be non-NULL");
+  if (a->x_stride < a->dim) return fail(MI_ERR_STRIDE, "x row stride %lld < dim", (long long)a->x_stride);
+  if (!backward) {
+    if (!a->y) return fail(MI_ERR_NULL_POINTER, "y must be non-NULL");
+    if (a->y_stride < a->dim) return fail(MI_ERR_STRIDE, "y row stride %lld < dim", (long long)a->y_stride);
+  } else {
+    if (!a->dy || !a->dx || !a->dw) return fail(MI_ERR_NULL_POINTER, "dy, dx and dw must be non-NULL");
+    if (a->dy_stride < a->dim || a->dx_stride < a->dim) return fail(MI_ERR_STRIDE, "dy / dx row stride < dim");
+    if (!a->workspace || a->workspace_bytes < mi_rmsnorm_bwd_workspace_bytes(a))
+      return fail(MI_ERR_WORKSPACE, "workspace of %zu bytes needed", mi_rmsnorm_bwd_workspace_bytes(a));
+  }
+  return MI_OK;
+}
+
+// 16-byte chunk path: dim and row strides multiples of the chunk, 16-byte aligned bases, <= 16 chunks per lane
+static bool rms_vec_ok(const mi_rmsnorm_args* a, bool backward) {
+  const int epc = 16 / rms_elem_bytes(a->x_dtype);
+  // chunks per row: 16 per thread of a workgroup; 8 in the backward pass, whose
+  // per-position dw sums share the registers
+  if (a->dim % epc || a->dim / epc > 256 * (backward ? 8 : 16)) return false;
+  if (!aligned16(a->x) || a->x_stride % epc) return false;
+  if (!backward) return aligned16(a->y) && a->y_stride % epc == 0;
+  return aligned16(a->dy) && aligned16(a->dx) && a->dy_stride % epc == 0 && a->dx_stride % epc == 0;
+}
+
+static void rms_fill(const mi_rmsnorm_args* a, mi::RmsParams& p) {
+  std::memset(&p, 0, sizeof(p));
+  p.x = a->x; p.w = a->w; p.dy = a->dy; p.y = a->y; p.dx = a->dx; p.dw = a->dw;
+  p.rsqrt = a->rsqrt; p.dw_part = static_cast<float*>(a->workspace);
+  p.x_st = a->x_stride; p.y_st = a->y_stride; p.dy_st = a->dy_stride; p.dx_st = a->dx_stride;
+  p.rows = a->rows; p.dim = a->dim; p.eps = a->eps;
+}
+
+int mi_rmsnorm_fwd(const mi_rmsnorm_args* a, void* stream) {
+  int rc = rms_validate(a, false);
+  if (rc) return rc;
+  if (a->rows == 0) return MI_OK;
+  mi::RmsParams p;
+  rms_fill(a, p);
+  return launch_status(mi::launch_rms_fwd(p, a->x_dtype, a->w_dtype, rms_vec_ok(a, false), mi::rms_partial_rows(a->rows, 256),
+                                          static_cast<hipStream_t>(stream)),
+                       "mi_rmsnorm_fwd");
+}
+
+size_t mi_rmsnorm_bwd_workspace_bytes(const mi_rmsnorm_args* a) {
+  if (!a || a->dim <= 0 || a->rows <= 0) return 0;
+  return (size_t)(mi::rms_partial_rows(a->rows, 256) + mi::kRmsStageRows) * (size_t)a->dim * sizeof(float);
+}
+
+int mi_rmsnorm_bwd(const mi_rmsnorm_args* a, void* stream) {
+  int rc = rms_validate(a, true);
+  if (rc) return rc;
+  if (a->rows == 0) return MI_OK;   // dw of an empty batch is left to the caller
+  mi::RmsParams p;
+  rms_fill(a, p);
+  return launch_status(mi::launch_rms_bwd(p, a->x_dtype, a->w_dtype, rms_vec_ok(a, true), mi::rms_partial_rows(a->rows, 256),
+                                          static_cast<hipStream_t>(stream)),
+                       "mi_rmsnorm_bwd");
+}
+
 int mi_attn_bwd_validate(const mi_attn_bwd_args* a) {
   if (!a) return fail(MI_ERR_NULL_POINTER, "args is NULL");
   if (a->struct_size != sizeof(mi_attn_bwd_args))
@@ -388,7 +462,7 @@ int mi_decode(const mi_decode_args* a, void* stream) {
 
 int mi_time_launches(int kind, const void* args, void* stream, int warmup, int iters, float* ms_per_launch) {
   if (!args || !ms_per_launch) return fail(MI_ERR_NULL_POINTER, "args / ms_per_launch is NULL");
-  if (iters <= 0 || warmup < 0 || kind < 0 || kind > 5) return fail(MI_ERR_SHAPE, "bad kind / warmup / iters");
+  if (iters <= 0 || warmup < 0 || kind < 0 || kind > 7) return fail(MI_ERR_SHAPE, "bad kind / warmup / iters");
   auto once = [&]() -> int {
     switch (kind) {
       case 0: return mi_attn_fwd(static_cast<const mi_attn_fwd_args*>(args), stream);
@@ -396,6 +470,8 @@ int mi_time_launches(int kind, const void* args, void* stream, int warmup, int i
       case 2: return mi_decode(static_cast<const mi_decode_args*>(args), stream);
       case 3: return mi_decode_splitkv(static_cast<const mi_decode_args*>(args), stream);
       case 5: return mi_attn_bwd(static_cast<const mi_attn_bwd_args*>(args), stream);
+      case 6: return mi_rmsnorm_fwd(static_cast<const mi_rmsnorm_args*>(args), stream);
+      case 7: return mi_rmsnorm_bwd(static_cast<const mi_rmsnorm_args*>(args), stream);
       default: return mi_decode_merge(static_cast<const mi_decode_args*>(args), stream);
     }
   };

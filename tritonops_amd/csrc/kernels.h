@@ -81,6 +81,17 @@ struct BwdParams {
   float scale_nat;    // natural base (= scale * ln 2)
 };
 
+struct RmsParams {
+  const void *x, *w, *dy;
+  void *y, *dx, *dw;
+  float* rsqrt;    // [rows] fp32: written by the forward, read by the backward
+  float* dw_part;  // workspace [partial rows][dim] fp32
+  int64_t x_st, y_st, dy_st, dx_st;  // row strides, elements
+  int64_t rows;
+  int32_t dim;
+  float eps;
+};
+
 // dtype: 0 bf16, 1 f16.  head_dim in {64, 96, 128}.  Return hipError_t as int.
 int launch_prefill_dense(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);
 int launch_prefill_sparse(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);
@@ -88,6 +99,15 @@ int launch_decode_splitkv(const DecodeParams& p, int dtype, int head_dim, hipStr
 int launch_decode_merge(const DecodeParams& p, int dtype, int head_dim, hipStream_t s);
 // delta, dq, dk, dv kernels in that order
 int launch_attn_bwd(const BwdParams& p, int dtype, int head_dim, hipStream_t s);
+// RMSNorm.  x_dtype: 0 bf16, 1 f16, 2 f32; w_dtype: x_dtype or 2.  `vec`: rows
+// can be read in 16-byte chunks (dim a multiple of the chunk, aligned rows,
+// at most 4096 chunks).  `n_waves` = rms_partial_rows(): wavefronts of the
+// launch and upper bound of the partial dw rows the backward pass writes.
+// The backward workspace holds rms_partial_rows() + kRmsStageRows fp32 rows of `dim`.
+constexpr int kRmsStageRows = 32;
+int rms_partial_rows(long long rows, int num_cus);
+int launch_rms_fwd(const RmsParams& p, int x_dtype, int w_dtype, bool vec, int n_waves, hipStream_t s);
+int launch_rms_bwd(const RmsParams& p, int x_dtype, int w_dtype, bool vec, int n_waves, hipStream_t s);
 
 // Query rows per workgroup of the two prefill kernels.
 constexpr int kDenseRows = 256;
