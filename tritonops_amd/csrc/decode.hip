@@ -128,8 +128,8 @@ decode_splitkv_kernel(const DecodeParams p) {
         const int row = idx / G::NCH, ch = idx % G::NCH;
         // rows past the end re-read the last token (same tile, hence same page)
         const int64_t kr = min(tb + row, len - 1);
-        kreg[i] = *reinterpret_cast<const i32x4*>(kp + kshift + kr * p.k_ss + ch * 8);
-        vreg[i] = *reinterpret_cast<const i32x4*>(vp + vshift + kr * p.v_ss + ch * 8);
+        kreg[i] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(kp + kshift + kr * p.k_ss + ch * 8));
+        vreg[i] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(vp + vshift + kr * p.v_ss + ch * 8));
       }
     }
   };

@@ -50,11 +50,16 @@ template <typename T, int J, int GROUP>
 struct RowRegs {
   static constexpr int EPC = Chunk<T>::EPC;
   Chunk<T> c[J];
+  // STREAM: the row is not read again soon (non-temporal hint)
+  template <bool STREAM = false>
   __device__ __forceinline__ void load(const T* row, int t, int nch) {
 #pragma unroll
     for (int j = 0; j < J; ++j) {
       const int ch = t + GROUP * j;
-      if (ch < nch) c[j].raw = *reinterpret_cast<const i32x4*>(row + ch * EPC);
+      if (ch < nch) {
+        const i32x4* src = reinterpret_cast<const i32x4*>(row + ch * EPC);
+        c[j].raw = STREAM ? __builtin_nontemporal_load(src) : *src;
+      }
     }
   }
 };
@@ -119,7 +124,7 @@ __global__ void __launch_bounds__(256) rms_fwd_vec_kernel(const RmsParams p) {
         Chunk<T> o;
 #pragma unroll
         for (int e = 0; e < EPC; ++e) o.set(e, cur.c[j].at(e) * r * (float)w[ch * EPC + e]);
-        *reinterpret_cast<i32x4*>(y + ch * EPC) = o.raw;
+        __builtin_nontemporal_store(o.raw, reinterpret_cast<i32x4*>(y + ch * EPC));
       }
     }
     if (t == 0) p.rsqrt[row] = r;
@@ -179,18 +184,18 @@ __global__ void __launch_bounds__(256) rms_bwd_vec_kernel(const RmsParams p) {
     for (int e = 0; e < EPC; ++e) dwacc[j][e] = 0.f;
   RowRegs<T, J, GROUP> cx, cd, nx, nd;
   if (PF && slot < p.rows) {
-    cx.load(xb + (int64_t)slot * p.x_st, t, nch);
-    cd.load(db + (int64_t)slot * p.dy_st, t, nch);
+    cx.template load<true>(xb + (int64_t)slot * p.x_st, t, nch);
+    cd.template load<true>(db + (int64_t)slot * p.dy_st, t, nch);
   }
   for (int64_t row = slot; row < p.rows; row += n_slots) {
     if (PF) {
       if (row + n_slots < p.rows) {
-        nx.load(xb + (row + n_slots) * p.x_st, t, nch);
-        nd.load(db + (row + n_slots) * p.dy_st, t, nch);
+        nx.template load<true>(xb + (row + n_slots) * p.x_st, t, nch);
+        nd.template load<true>(db + (row + n_slots) * p.dy_st, t, nch);
       }
     } else {
-      cx.load(xb + row * p.x_st, t, nch);
-      cd.load(db + row * p.dy_st, t, nch);
+      cx.template load<true>(xb + row * p.x_st, t, nch);
+      cd.template load<true>(db + row * p.dy_st, t, nch);
     }
     T* dx = reinterpret_cast<T*>(p.dx) + row * p.dx_st;
     const float r = p.rsqrt[row];
@@ -216,7 +221,7 @@ __global__ void __launch_bounds__(256) rms_bwd_vec_kernel(const RmsParams p) {
           o.set(e, dv * (float)w[ch * EPC + e] * r - xv * k);
           dwacc[j][e] += dv * xv * r;
         }
-        *reinterpret_cast<i32x4*>(dx + ch * EPC) = o.raw;
+        __builtin_nontemporal_store(o.raw, reinterpret_cast<i32x4*>(dx + ch * EPC));
       }
     }
     if (PF) {
