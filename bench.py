@@ -358,6 +358,42 @@ def run_rmsnorm(steps, warmup):
     }
 
 
+def run_fused_xent(steps, warmup):
+    """Fused linear + cross-entropy, Llama-3-sized head: 8192 tokens, hidden 4096, vocabulary 128256."""
+    import tritonops_amd as ta
+    from tritonops_amd import _lib
+    T, D, N = 8192, 4096, 128256
+    x = _randn((T, D), 0)
+    w = (_randn((N, D), 1).float() * (D ** -0.5)).to(torch.bfloat16)
+    y = torch.randint(0, N, (T,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(2))
+    steps, warmup = max(steps // 4, 3), max(warmup // 4, 2)
+    ms = _time_steps(lambda: ta.cross_entropy_fused_fwd(x, w, y), steps, warmup)
+    loss, lse = ta.cross_entropy_fused_fwd(x, w, y)
+    go = torch.full((T,), 1.0 / T, device="cuda")
+    ms_bwd = _time_steps(lambda: ta.cross_entropy_fused_bwd(go, x, w, y, lse), max(steps // 2, 2), 1)
+    a = _lib.XentArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype, a.tokens, a.dim, a.vocab, a.labels_i64 = _lib.MI_DTYPE_BF16, T, D, N, 1
+    a.x, a.w, a.y, a.lse, a.loss = x.data_ptr(), w.data_ptr(), y.data_ptr(), lse.data_ptr(), loss.data_ptr()
+    a.x_stride = a.w_stride = D
+    nb = _lib.load().mi_xent_fwd_workspace_bytes(C.byref(a))
+    ws = torch.empty(nb, device="cuda", dtype=torch.uint8)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), nb
+    kms = _event_ms(8, a, steps, warmup)
+    flop = 2.0 * T * D * N
+    return {
+        "name": "fused_xent", "ms_per_step": ms, "kernel_ms": kms,
+        "metric": "fused_linear_xent_fwd_tflops", "unit": "TFLOP/s", "value": flop / (ms * 1e-3) / 1e12,
+        "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "kernel": "xent_fwd_kernel<bf16> (+ combine)"},
+        "config": {"workload": "fused linear + cross-entropy forward bf16, T=8192 tokens, hidden 4096, vocabulary 128256",
+                   "flop_per_step": flop, "bwd_ms_per_step": ms_bwd,
+                   "bwd_note": "backward = logits GEMM + in-place dlogits kernel + two gradient GEMMs (6*T*D*N FLOP, "
+                               "library GEMMs through torch.mm)",
+                   "bwd_tflops": 3.0 * flop / (ms_bwd * 1e-3) / 1e12},
+    }
+
+
 WORKLOADS = {
     "dense_causal": run_dense_causal,
     "gqa_decode": run_decode,
@@ -365,6 +401,7 @@ WORKLOADS = {
     "sparse_decode": run_sparse_decode,
     "dense_causal_bwd": run_dense_bwd,
     "rmsnorm": run_rmsnorm,
+    "fused_xent": run_fused_xent,
 }
 
 
@@ -435,6 +472,21 @@ def cpu_baseline(name):
                 "sample": "torch-CPU RMSNorm forward (fp32 math, bf16 result) + float64 backward formulas of the oracle "
                           "(common/rms.py math) on [4096, 4096] bf16 (1/8 of the rows), median of 3; same "
                           "algorithmic-byte formula as the GPU figure",
+                "seconds": t}
+    if name == "fused_xent":
+        from oracle import xent_oracle as xo
+        T, D, N = 128, 4096, 128256
+        x = torch.randn((T, D), generator=g).to(torch.bfloat16)
+        w = (torch.randn((N, D), generator=g) * D ** -0.5).to(torch.bfloat16)
+        y = torch.randint(0, N, (T,), generator=g)
+
+        def fn():
+            logits = (x @ w.t()).float()
+            return torch.logsumexp(logits, -1) - logits.gather(-1, y.view(-1, 1)).squeeze(-1)
+        t = med(fn)
+        return {"value": 2.0 * T * D * N / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "sample": "torch-CPU bf16 x @ w^T, fp32 logsumexp - target logit (cross_entropy.py:428-435 math) on 128 of "
+                          "the 8192 tokens, median of 3; same FLOP formula as the GPU figure",
                 "seconds": t}
     return None
 

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define MI_ATTN_ABI_VERSION 2
+#define MI_ATTN_ABI_VERSION 3
 
 /* KV tile edge (tokens) of the prefill kernels and block edge of the block
  * sparse layouts; fixed at build time. */
@@ -331,6 +331,56 @@ size_t mi_rmsnorm_bwd_workspace_bytes(const mi_rmsnorm_args *args);
 int mi_rmsnorm_bwd(const mi_rmsnorm_args *args, void *stream);
 
 /* ------------------------------------------------------------------------- */
+/* Fused linear + cross-entropy.
+ *
+ * Replaces CrossEntropyFusedFunction.forward and its kernel
+ * cross_entropy_fused_fwd_lse_kernel (cross_entropy_triton/cross_entropy.py:
+ * 276-352, :43-183) and the element-wise kernel of its backward
+ * (cross_entropy_fused_bwd_kernel, :185-266):
+ *   logits[t,n] = sum_d x[t,d] w[n,d]             (never written by the forward)
+ *   lse[t]      = log sum_n exp(logits[t,n])       fp32, saved for the backward
+ *   loss[t]     = lse[t] - logits[t, y[t]]         fp32
+ *   dlogits[t,n] = dloss[t] (exp(logits[t,n] - lse[t]) - [n == y[t]])
+ * x [tokens, dim] and w [vocab, dim] are bf16 or f16, row-major with row
+ * strides in elements (multiples of 8, bases 16-byte aligned); dim must be a
+ * multiple of 128 (pad x and w with zero columns otherwise).  Labels are int32
+ * or int64; a label outside [0, vocab) contributes no target logit
+ * (loss = lse).  The forward needs mi_xent_fwd_workspace_bytes() of device
+ * workspace for the per-range partial results.
+ */
+typedef struct mi_xent_args {
+  uint32_t struct_size;
+  int32_t dtype;                 /* of x and w                                 */
+  int32_t tokens, dim, vocab;
+  int32_t labels_i64;            /* 1: y is int64, 0: int32                    */
+  const void *x, *w;             /* device                                     */
+  const void *y;                 /* [tokens] labels                            */
+  int64_t x_stride, w_stride;    /* row strides, elements                      */
+  float *lse, *loss;             /* [tokens] fp32 outputs                      */
+  void *workspace;
+  size_t workspace_bytes;
+} mi_xent_args;
+
+size_t mi_xent_fwd_workspace_bytes(const mi_xent_args *args);
+int mi_xent_fwd(const mi_xent_args *args, void *stream);
+
+/* In place over a block of logits [rows, vocab] (row stride ld, elements):
+ * logits[t,n] <- dloss[t] (exp(logits[t,n] - lse[t]) - [n == y[t]]), the
+ * operand of the two gradient GEMMs (cross_entropy.py:255-266, :369-415). */
+typedef struct mi_xent_grad_args {
+  uint32_t struct_size;
+  int32_t dtype;                 /* of logits                                  */
+  int32_t vocab;
+  int32_t labels_i64;
+  int64_t rows, ld;
+  void *logits;                  /* device, in / out                           */
+  const float *lse, *dloss;      /* [rows] fp32                                */
+  const void *y;                 /* [rows] labels                              */
+} mi_xent_grad_args;
+
+int mi_xent_dlogits(const mi_xent_grad_args *args, void *stream);
+
+/* ------------------------------------------------------------------------- */
 /* Introspection (host only). */
 int mi_abi_version(void);
 /* Message of the last failing call on this thread ("" if none). */
@@ -348,7 +398,8 @@ int mi_attn_bwd_validate(const mi_attn_bwd_args *args);
  * untimed ones).  Blocks the calling thread; for benchmarking only.
  * kind: 0 = mi_attn_fwd, 1 = mi_attn_fwd_blocksparse, 2 = mi_decode,
  *       3 = mi_decode_splitkv, 4 = mi_decode_merge, 5 = mi_attn_bwd,
- *       6 = mi_rmsnorm_fwd, 7 = mi_rmsnorm_bwd.
+ *       6 = mi_rmsnorm_fwd, 7 = mi_rmsnorm_bwd, 8 = mi_xent_fwd,
+ *       9 = mi_xent_dlogits.
  * Returns MI_OK and writes milliseconds to *ms_per_launch. */
 int mi_time_launches(int kind, const void *args, void *stream, int warmup,
                      int iters, float *ms_per_launch);

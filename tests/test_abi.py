@@ -27,17 +27,19 @@ def test_every_declared_symbol_is_exported(lib):
     assert declared == set(_lib.EXPORTS), "ctypes table and header disagree: %s" % (declared ^ set(_lib.EXPORTS))
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.mi_abi_version() == _lib.MI_ATTN_ABI_VERSION == 2
+    assert lib.mi_abi_version() == _lib.MI_ATTN_ABI_VERSION == 3
 
 
 def test_struct_layout_matches_the_c_compiler(tmp_path):
     src = tmp_path / "sz.c"
-    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "mi_attn.h"\nint main(){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\\n",'
+    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "mi_attn.h"\nint main(){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\\n",'
                    "sizeof(mi_attn_fwd_args),sizeof(mi_attn_sparse_args),sizeof(mi_decode_args),"
                    "offsetof(mi_attn_fwd_args,scale_log2),offsetof(mi_attn_sparse_args,scale_log2),"
                    "offsetof(mi_decode_args,page_table),"
                    "sizeof(mi_attn_bwd_args),offsetof(mi_attn_bwd_args,workspace),"
-                   "sizeof(mi_rmsnorm_args),offsetof(mi_rmsnorm_args,eps));return 0;}\n")
+                   "sizeof(mi_rmsnorm_args),offsetof(mi_rmsnorm_args,eps),"
+                   "sizeof(mi_xent_args),offsetof(mi_xent_args,workspace),"
+                   "sizeof(mi_xent_grad_args),offsetof(mi_xent_grad_args,y));return 0;}\n")
     exe = tmp_path / "sz"
     subprocess.check_call(["gcc", "-std=c99", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
     got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
@@ -45,7 +47,9 @@ def test_struct_layout_matches_the_c_compiler(tmp_path):
             _lib.AttnFwdArgs.scale_log2.offset, _lib.AttnSparseArgs.scale_log2.offset,
             _lib.DecodeArgs.page_table.offset,
             C.sizeof(_lib.AttnBwdArgs), _lib.AttnBwdArgs.workspace.offset,
-            C.sizeof(_lib.RmsNormArgs), _lib.RmsNormArgs.eps.offset]
+            C.sizeof(_lib.RmsNormArgs), _lib.RmsNormArgs.eps.offset,
+            C.sizeof(_lib.XentArgs), _lib.XentArgs.workspace.offset,
+            C.sizeof(_lib.XentGradArgs), _lib.XentGradArgs.y.offset]
     assert got == want
 
 
@@ -250,6 +254,46 @@ def test_backward_and_rmsnorm_validation(lib):
     assert lib.mi_rmsnorm_fwd(C.byref(r), None) == 0 and lib.mi_rmsnorm_bwd(C.byref(r), None) == 0
 
 
+def test_fused_cross_entropy_validation(lib):
+    a = _lib.XentArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype, a.tokens, a.dim, a.vocab, a.labels_i64 = 0, 8192, 4096, 128256, 1
+    a.x = a.w = a.y = a.lse = a.loss = 0x1000
+    a.x_stride = a.w_stride = 4096
+    # 32 token tiles of 256 -> 8 vocabulary ranges fill 256 CUs; two fp32 per token and range
+    assert lib.mi_xent_fwd_workspace_bytes(C.byref(a)) == 8192 * 8 * 2 * 4
+    # a launch would follow a clean validation, so only the failing cases are called here
+    assert lib.mi_status_name(lib.mi_xent_fwd(C.byref(a), None)).decode() == "MI_ERR_WORKSPACE"
+    a.workspace, a.workspace_bytes = 0x2000, 1 << 20
+    a.dim = 4000
+    assert lib.mi_status_name(lib.mi_xent_fwd(C.byref(a), None)).decode() == "MI_ERR_SHAPE"
+    a.dim, a.x_stride = 4096, 4000
+    assert lib.mi_status_name(lib.mi_xent_fwd(C.byref(a), None)).decode() == "MI_ERR_STRIDE"
+    a.x_stride, a.dtype = 4096, 2
+    assert lib.mi_status_name(lib.mi_xent_fwd(C.byref(a), None)).decode() == "MI_ERR_DTYPE"
+    a.dtype, a.x = 0, 0x1008
+    assert lib.mi_status_name(lib.mi_xent_fwd(C.byref(a), None)).decode() == "MI_ERR_ALIGNMENT"
+    a.x, a.loss = 0x1000, None
+    assert lib.mi_status_name(lib.mi_xent_fwd(C.byref(a), None)).decode() == "MI_ERR_NULL_POINTER"
+    a.tokens = 0
+    assert lib.mi_xent_fwd(C.byref(a), None) == 0
+    # few tokens: one token tile, as many ranges as CUs, never more than vocabulary tiles
+    a.tokens, a.vocab = 100, 1000
+    assert lib.mi_xent_fwd_workspace_bytes(C.byref(a)) == 100 * 4 * 2 * 4
+
+    g = _lib.XentGradArgs()
+    g.struct_size = C.sizeof(g)
+    g.dtype, g.vocab, g.labels_i64, g.rows, g.ld = 0, 1000, 1, 16, 900
+    g.logits = g.lse = g.dloss = g.y = 0x1000
+    assert lib.mi_status_name(lib.mi_xent_dlogits(C.byref(g), None)).decode() == "MI_ERR_STRIDE"
+    g.ld, g.y = 1000, None
+    assert lib.mi_status_name(lib.mi_xent_dlogits(C.byref(g), None)).decode() == "MI_ERR_NULL_POINTER"
+    g.rows = 0
+    assert lib.mi_xent_dlogits(C.byref(g), None) == 0
+    g.struct_size = 4
+    assert lib.mi_xent_dlogits(C.byref(g), None) == -2
+
+
 def test_split_blocks_heuristic(lib):
     f = lib.mi_decode_choose_split_blocks
     # 32 sequences x 8 kv-heads on 256 CUs: 2048 resident wavefronts / 256 units = 8 chunks of 129 blocks
@@ -267,7 +311,7 @@ def test_time_launches_rejects_bad_arguments(lib):
     ms = C.c_float()
     assert lib.mi_time_launches(0, None, None, 0, 1, C.byref(ms)) == -1
     a = _good_fwd()
-    assert lib.mi_time_launches(9, C.cast(C.byref(a), C.c_void_p), None, 0, 1, C.byref(ms)) == -6
+    assert lib.mi_time_launches(10, C.cast(C.byref(a), C.c_void_p), None, 0, 1, C.byref(ms)) == -6
     a.head_dim = 5
     assert lib.mi_time_launches(0, C.cast(C.byref(a), C.c_void_p), None, 1, 1, C.byref(ms)) == -4
 

@@ -11,4 +11,11 @@ from .ops import (  # noqa: F401
     flash_attn_triton_fwd,
 )
 from .rms import RMSNormTriton, RMSNormTritonFunction, rmsnorm_bwd, rmsnorm_fwd  # noqa: F401
+from .xent import (  # noqa: F401
+    CrossEntropyFusedFunction,
+    cross_entropy_dlogits_,
+    cross_entropy_fused_bwd,
+    cross_entropy_fused_fwd,
+    cross_entropy_fused_triton,
+)
 from . import masks  # noqa: F401

@@ -229,6 +229,68 @@ int mi_rmsnorm_bwd(const mi_rmsnorm_args* a, void* stream) {
                        "mi_rmsnorm_bwd");
 }
 
+static int xent_validate(const mi_xent_args* a) {
+  if (!a) return fail(MI_ERR_NULL_POINTER, "args is NULL");
+  if (a->struct_size != sizeof(mi_xent_args))
+    return fail(MI_ERR_STRUCT_SIZE, "mi_xent_args.struct_size %u != %zu", a->struct_size, sizeof(mi_xent_args));
+  if (a->dtype != MI_DTYPE_BF16 && a->dtype != MI_DTYPE_F16) return fail(MI_ERR_DTYPE, "dtype %d is not bf16 / f16", a->dtype);
+  if (a->tokens < 0 || a->dim <= 0 || a->vocab <= 0)
+    return fail(MI_ERR_SHAPE, "tokens %d must be >= 0, dim %d and vocab %d positive", a->tokens, a->dim, a->vocab);
+  if (a->dim % 128) return fail(MI_ERR_SHAPE, "dim %d must be a multiple of 128 (pad with zero columns)", a->dim);
+  if (a->labels_i64 != 0 && a->labels_i64 != 1) return fail(MI_ERR_SHAPE, "labels_i64 must be 0 or 1");
+  if (a->tokens == 0) return MI_OK;
+  if (!a->x || !a->w || !a->y || !a->lse || !a->loss)
+    return fail(MI_ERR_NULL_POINTER, "x, w, y, lse and loss must be non-NULL");
+  if (!aligned16(a->x) || !aligned16(a->w)) return fail(MI_ERR_ALIGNMENT, "x and w must be 16-byte aligned");
+  if (a->x_stride < a->dim || a->w_stride < a->dim || a->x_stride % 8 || a->w_stride % 8)
+    return fail(MI_ERR_STRIDE, "row strides must be >= dim and multiples of 8 elements");
+  // per-lane row offsets inside a 256-row slab are 32-bit
+  if (a->x_stride > (1 << 22) || a->w_stride > (1 << 22)) return fail(MI_ERR_STRIDE, "row stride beyond 2^22 elements");
+  if (!a->workspace || a->workspace_bytes < mi_xent_fwd_workspace_bytes(a))
+    return fail(MI_ERR_WORKSPACE, "workspace of %zu bytes needed", mi_xent_fwd_workspace_bytes(a));
+  return MI_OK;
+}
+
+size_t mi_xent_fwd_workspace_bytes(const mi_xent_args* a) {
+  if (!a || a->tokens <= 0 || a->vocab <= 0) return 0;
+  return (size_t)a->tokens * (size_t)mi::xent_choose_splits(a->tokens, a->vocab, 256) * 2 * sizeof(float);
+}
+
+int mi_xent_fwd(const mi_xent_args* a, void* stream) {
+  int rc = xent_validate(a);
+  if (rc) return rc;
+  if (a->tokens == 0) return MI_OK;
+  mi::XentParams p;
+  std::memset(&p, 0, sizeof(p));
+  p.x = a->x; p.w = a->w; p.y = a->y; p.y_is_i64 = a->labels_i64;
+  p.x_st = a->x_stride; p.w_st = a->w_stride;
+  p.T = a->tokens; p.D = a->dim; p.N = a->vocab;
+  p.n_split = mi::xent_choose_splits(a->tokens, a->vocab, 256);
+  p.lse_part = static_cast<float*>(a->workspace);
+  p.tgt_part = p.lse_part + (size_t)a->tokens * p.n_split;
+  p.lse = a->lse; p.loss = a->loss;
+  return launch_status(mi::launch_xent_fwd(p, a->dtype, static_cast<hipStream_t>(stream)), "mi_xent_fwd");
+}
+
+int mi_xent_dlogits(const mi_xent_grad_args* a, void* stream) {
+  if (!a) return fail(MI_ERR_NULL_POINTER, "args is NULL");
+  if (a->struct_size != sizeof(mi_xent_grad_args))
+    return fail(MI_ERR_STRUCT_SIZE, "mi_xent_grad_args.struct_size %u != %zu", a->struct_size, sizeof(mi_xent_grad_args));
+  if (a->dtype != MI_DTYPE_BF16 && a->dtype != MI_DTYPE_F16) return fail(MI_ERR_DTYPE, "dtype %d is not bf16 / f16", a->dtype);
+  if (a->rows < 0 || a->vocab <= 0 || a->rows > 0x7fffffffLL)
+    return fail(MI_ERR_SHAPE, "rows %lld must be in [0, 2^31), vocab %d positive", (long long)a->rows, a->vocab);
+  if (a->labels_i64 != 0 && a->labels_i64 != 1) return fail(MI_ERR_SHAPE, "labels_i64 must be 0 or 1");
+  if (a->rows == 0) return MI_OK;
+  if (!a->logits || !a->lse || !a->dloss || !a->y) return fail(MI_ERR_NULL_POINTER, "logits, lse, dloss and y must be non-NULL");
+  if (a->ld < a->vocab) return fail(MI_ERR_STRIDE, "ld %lld < vocab", (long long)a->ld);
+  mi::XentGradParams p;
+  std::memset(&p, 0, sizeof(p));
+  p.logits = a->logits; p.lse = a->lse; p.dloss = a->dloss; p.y = a->y;
+  p.ld = a->ld; p.rows = a->rows; p.N = a->vocab; p.y_is_i64 = a->labels_i64;
+  p.vec = aligned16(a->logits) && a->ld % 8 == 0;
+  return launch_status(mi::launch_xent_dlogits(p, a->dtype, static_cast<hipStream_t>(stream)), "mi_xent_dlogits");
+}
+
 int mi_attn_bwd_validate(const mi_attn_bwd_args* a) {
   if (!a) return fail(MI_ERR_NULL_POINTER, "args is NULL");
   if (a->struct_size != sizeof(mi_attn_bwd_args))
@@ -462,7 +524,7 @@ int mi_decode(const mi_decode_args* a, void* stream) {
 
 int mi_time_launches(int kind, const void* args, void* stream, int warmup, int iters, float* ms_per_launch) {
   if (!args || !ms_per_launch) return fail(MI_ERR_NULL_POINTER, "args / ms_per_launch is NULL");
-  if (iters <= 0 || warmup < 0 || kind < 0 || kind > 7) return fail(MI_ERR_SHAPE, "bad kind / warmup / iters");
+  if (iters <= 0 || warmup < 0 || kind < 0 || kind > 9) return fail(MI_ERR_SHAPE, "bad kind / warmup / iters");
   auto once = [&]() -> int {
     switch (kind) {
       case 0: return mi_attn_fwd(static_cast<const mi_attn_fwd_args*>(args), stream);
@@ -472,6 +534,8 @@ int mi_time_launches(int kind, const void* args, void* stream, int warmup, int i
       case 5: return mi_attn_bwd(static_cast<const mi_attn_bwd_args*>(args), stream);
       case 6: return mi_rmsnorm_fwd(static_cast<const mi_rmsnorm_args*>(args), stream);
       case 7: return mi_rmsnorm_bwd(static_cast<const mi_rmsnorm_args*>(args), stream);
+      case 8: return mi_xent_fwd(static_cast<const mi_xent_args*>(args), stream);
+      case 9: return mi_xent_dlogits(static_cast<const mi_xent_grad_args*>(args), stream);
       default: return mi_decode_merge(static_cast<const mi_decode_args*>(args), stream);
     }
   };

@@ -92,6 +92,30 @@ struct RmsParams {
   float eps;
 };
 
+struct XentParams {
+  const void *x, *w;   // [T, D], [N, D] row-major, row strides in elements
+  const void* y;       // [T] int32 or int64 labels
+  float* lse_part;     // workspace [T][n_split]
+  float* tgt_part;     // workspace [T][n_split]
+  float *lse, *loss;   // [T]
+  int64_t x_st, w_st;
+  int32_t T, D, N;
+  int32_t y_is_i64;
+  int32_t n_split;           // vocabulary ranges (xent_choose_splits)
+  int32_t tiles_t, block_t;  // set by the launcher
+};
+
+struct XentGradParams {
+  void* logits;        // [rows, N] in / dlogits out, row stride ld (elements)
+  const float* lse;    // [rows]
+  const float* dloss;  // [rows]
+  const void* y;
+  int64_t ld, rows;
+  int32_t N;
+  int32_t y_is_i64;
+  int32_t vec;         // rows can be accessed in 16-byte chunks
+};
+
 // dtype: 0 bf16, 1 f16.  head_dim in {64, 96, 128}.  Return hipError_t as int.
 int launch_prefill_dense(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);
 int launch_prefill_sparse(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);
@@ -108,6 +132,11 @@ constexpr int kRmsStageRows = 32;
 int rms_partial_rows(long long rows, int num_cus);
 int launch_rms_fwd(const RmsParams& p, int x_dtype, int w_dtype, bool vec, int n_waves, hipStream_t s);
 int launch_rms_bwd(const RmsParams& p, int x_dtype, int w_dtype, bool vec, int n_waves, hipStream_t s);
+
+// Fused linear + cross-entropy.  D a multiple of 64, rows 16-byte aligned.
+int xent_choose_splits(long long tokens, int vocab, int num_cus);
+int launch_xent_fwd(const XentParams& p, int dtype, hipStream_t s);       // partials + combine
+int launch_xent_dlogits(const XentGradParams& p, int dtype, hipStream_t s);
 
 // Query rows per workgroup of the two prefill kernels.
 constexpr int kDenseRows = 256;
