@@ -94,3 +94,28 @@ def test_strided_rows_and_determinism():
     a = ta.rmsnorm_bwd(dy, x, w, rs, 1e-6)
     b = ta.rmsnorm_bwd(dy, x, w, rs, 1e-6)
     assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])   # no atomics: bit-reproducible
+
+
+def test_full_size_properties():
+    """Benchmark shape [32768, 4096] bf16: unit RMS of y / w, invariance of y to
+    a power-of-two scaling of x (eps = 0), dx orthogonal to x when w = 1."""
+    import tritonops_amd as ta
+
+    T, D = 32768, 4096
+    g = torch.Generator(device="cuda").manual_seed(9)
+    x = torch.randn((T, D), device="cuda", generator=g).to(torch.bfloat16)
+    dy = torch.randn((T, D), device="cuda", generator=g).to(torch.bfloat16)
+    w = torch.ones(D, device="cuda", dtype=torch.float32)
+    y, rs = ta.rmsnorm_fwd(x, w, 0.0)
+    rms = y.float().pow(2).mean(-1).sqrt()
+    assert (rms - 1).abs().max().item() < 3e-3            # bf16 rounding of 4096 outputs
+    y4, rs4 = ta.rmsnorm_fwd(x * 4, w, 0.0)
+    assert torch.equal(y4, y)                              # exact: scaling by 4 only moves exponents
+    assert torch.allclose(rs4 * 4, rs, rtol=1e-6, atol=0)
+    dx, dw = ta.rmsnorm_bwd(dy, x, w, rs, 0.0)
+    # d/dx of a scale-invariant function is orthogonal to x
+    dots = (dx.float() * x.float()).sum(-1)
+    scale = (dx.float().norm(dim=-1) * x.float().norm(dim=-1))
+    assert (dots.abs() / scale).max().item() < 2e-3
+    want_dw = (dy.float() * x.float() * rs.view(-1, 1)).sum(0)
+    assert (dw - want_dw).abs().max().item() <= 2e-2 * want_dw.abs().max().item()

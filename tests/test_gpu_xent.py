@@ -138,3 +138,29 @@ def test_dlogits_kernel_rows_and_tails():
     wide[:, :N] = logits
     got2 = ta.cross_entropy_dlogits_(wide.cuda()[:, :N], lse.cuda(), go.cuda(), y.cuda())
     assert torch.equal(got2.cpu(), got.cpu())
+
+
+def test_full_size_is_invariant_to_the_launch_shape():
+    """Benchmark shape (8192 tokens, hidden 4096, vocabulary 128256): the loss of
+    a token does not depend on how tokens and vocabulary are dealt to
+    workgroups.  8192 tokens run as 32 token tiles x 8 vocabulary ranges, a
+    slice of 1024 tokens as 4 x 64, a slice of 100 as 1 x 256."""
+    import tritonops_amd as ta
+
+    T, D, N = 8192, 4096, 128256
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn((T, D), device="cuda", generator=g).to(torch.bfloat16)
+    w = (torch.randn((N, D), device="cuda", generator=g) * D ** -0.5).to(torch.bfloat16)
+    y = torch.randint(0, N, (T,), device="cuda", generator=g)
+    loss, lse = ta.cross_entropy_fused_fwd(x, w, y)
+    assert torch.isfinite(loss).all() and (loss > 0).all()
+    # N(0,1) logits: lse = log N + 1/2 up to sampling noise
+    assert abs(lse.mean().item() - (math.log(N) + 0.5)) < 0.05
+    for lo, hi in ((3072, 4096), (8000, 8100)):
+        l2, s2 = ta.cross_entropy_fused_fwd(x[lo:hi], w, y[lo:hi])
+        assert (l2 - loss[lo:hi]).abs().max().item() <= 1e-4
+        assert (s2 - lse[lo:hi]).abs().max().item() <= 1e-4
+    # against fp32 torch math on a slice of tokens (same bf16 inputs, full vocabulary)
+    logits = x[:64].float() @ w.float().t()
+    want = torch.logsumexp(logits, -1) - logits.gather(-1, y[:64].view(-1, 1)).squeeze(-1)
+    assert (loss[:64] - want).abs().max().item() <= 2e-3
