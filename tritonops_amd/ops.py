@@ -51,6 +51,24 @@ def _max_len(cu_seq_lens, max_seq_len):
     return int((cu_seq_lens[1:] - cu_seq_lens[:-1]).max().item())
 
 
+_HEAD_DIMS = (64, 96, 128)
+
+
+def _padded_head_dim(D):
+    """Smallest head_dim the kernels are built for that holds D.  The reference
+    pads every head_dim to the next power of two inside its kernels
+    (flash_attn_triton.py:612); zero columns change neither q.k nor the first D
+    columns of the output."""
+    for d in _HEAD_DIMS:
+        if D <= d:
+            return d
+    raise ValueError("head_dim %d is not supported (at most %d)" % (D, _HEAD_DIMS[-1]))
+
+
+def _pad_last(t, Dp):
+    return t if t.shape[-1] == Dp else torch.nn.functional.pad(t, (0, Dp - t.shape[-1]))
+
+
 def _fill_qkvo(a, q, k, v, o, lse, packed):
     """q/k/v/o given as [X, S, H, D] views (X = 1 packed, X = B batched)."""
     a.q, a.k, a.v, a.o, a.lse = _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse)
@@ -75,6 +93,13 @@ def _dense_fwd(q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, want_lse=T
     X, S, Hq, D = q.shape
     if k.shape[-1] != D or v.shape[-1] != D:
         raise ValueError("q, k and v must share head_dim (got %d, %d, %d)" % (D, k.shape[-1], v.shape[-1]))
+    Dp = _padded_head_dim(D)
+    if Dp != D:
+        o, lse = _dense_fwd(_pad_last(q, Dp), _pad_last(k, Dp), _pad_last(v, Dp), cu_seq_lens, scale_log2, causal,
+                            max_seq_len, want_lse, bhsd)
+        if bhsd:
+            return o.transpose(1, 2)[..., :D].contiguous().transpose(1, 2), lse
+        return o[..., :D].contiguous(), lse
     if bhsd:
         o = torch.empty((X, Hq, S, D), device=q.device, dtype=q.dtype).transpose(1, 2)
         lse = torch.empty((X, Hq, S), device=q.device, dtype=torch.float32).transpose(1, 2) if want_lse else None
@@ -111,6 +136,11 @@ def _dense_bwd(q, k, v, o, lse, do, cu_seq_lens, scale_log2, causal, max_seq_len
     q, k, v, o, do = (_inner_contig(t) for t in (q, k, v, o, do))
     packed = cu_seq_lens is not None
     X, S, Hq, D = q.shape
+    Dp = _padded_head_dim(D)
+    if Dp != D:
+        grads = _dense_bwd(*(_pad_last(t, Dp) for t in (q, k, v, o)), lse, _pad_last(do, Dp), cu_seq_lens,
+                           scale_log2, causal, max_seq_len)
+        return tuple(g[..., :D].contiguous() for g in grads)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     a = _lib.AttnBwdArgs()
     a.struct_size = C.sizeof(a)
@@ -229,6 +259,14 @@ def flash_attn_sparse_triton(q, k, v, cu_seqlens, softmax_scale=None, local_wind
     """
     _require_gpu(q, k, v, cu_seqlens)
     lib = _lib.load()
+    D0 = q.shape[-1]
+    if _padded_head_dim(D0) != D0:
+        Dp = _padded_head_dim(D0)
+        o, lse = flash_attn_sparse_triton(
+            _pad_last(q, Dp), _pad_last(k, Dp), _pad_last(v, Dp), cu_seqlens,
+            D0 ** -0.5 if softmax_scale is None else softmax_scale, local_window_size, global_window_size,
+            block_mask=block_mask, row_ptr=row_ptr, col_idx=col_idx, csr_strides=csr_strides, max_seq_len=max_seq_len)
+        return o[..., :D0].contiguous(), lse
     q, k, v = _inner_contig(q), _inner_contig(k), _inner_contig(v)
     packed = cu_seqlens is not None
     if packed:
@@ -284,11 +322,22 @@ def _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, re
             window=(-1, -1), include_last=False, kv_layout="batched", page_table=None, page_size=0):
     _require_gpu(q, k, v, cu_seq_lens, seq_lens, page_table)
     lib = _lib.load()
+    if v.shape[-1] != q.shape[-1] or k.shape[-1] != q.shape[-1]:
+        raise ValueError("q, k and v must share head_dim")
+    D0 = q.shape[-1]
+    if _padded_head_dim(D0) != D0:
+        # zero-padded copies of the cache: correct, but a cache that is decoded from
+        # repeatedly should be allocated with a head_dim the kernels are built for
+        Dp = _padded_head_dim(D0)
+        out = _decode(_pad_last(q, Dp), _pad_last(k, Dp), _pad_last(v, Dp), cu_seq_lens, seq_lens, scale, max_seq_len,
+                      split_tokens, return_lse, block_idx, block_cnt, bi_strides, max_blocks, split_blocks, window,
+                      include_last, kv_layout, page_table, page_size)
+        if return_lse:
+            return out[0][..., :D0].contiguous(), out[1]
+        return out[..., :D0].contiguous()
     q, k, v = _inner_contig(q), _inner_contig(k), _inner_contig(v)
     B, Hq, D = q.shape
     Hkv = k.shape[2]
-    if v.shape[-1] != D or k.shape[-1] != D:
-        raise ValueError("q, k and v must share head_dim")
     o = torch.empty((B, Hq, D), device=q.device, dtype=q.dtype)
     lse = torch.empty((B, Hq), device=q.device, dtype=torch.float32) if return_lse else None
     a = _lib.DecodeArgs()
