@@ -110,6 +110,10 @@ decode_splitkv_kernel(const DecodeParams p) {
   for (int db = 0; db < G::NDB; ++db) O[db] = (f32x16){0};
   float m = -INFINITY, l = 0.f;
 
+  // The loads of tile t + 1 fly while tile t is worked on.  (Registers for a
+  // second tile in flight do not exist: the occupancy of this kernel is bounded
+  // by LDS, one private tile per wave, at 256 registers per wave, and O, Q and
+  // one K/V set already take 240 of them at head_dim 128.)
   i32x4 kreg[LOADS], vreg[LOADS];
   // First token a tile is fetched from.  A tile that is masked as a whole (a
   // dropped duplicate, base -1, or the second half of the last block when the
@@ -118,22 +122,62 @@ decode_splitkv_kernel(const DecodeParams p) {
   // sequence is ever touched.
   const int last_tile = ((len - 1) / kDecTile) * kDecTile;
   auto addr_base = [&](int base) -> int { return min(max(base, 0), last_tile); };
-  // kshift / vshift: page_shift() of the tile (0 unless paged)
-  auto gload = [&](int base, int64_t kshift, int64_t vshift) {
-    const int tb = addr_base(base);
+  // Load i of a lane covers chunk lane % NCH of row lane / NCH + i * (64 / NCH)
+  // when NCH divides 64 (head_dim 64 and 128): the address is then a uniform
+  // base that advances by a fixed step per load plus one 32-bit lane offset.
+  constexpr bool kUniformRows = 64 % G::NCH == 0;
+  typedef __attribute__((address_space(1))) const i32x4 g_i32x4;  // global memory, not generic
+  typedef __attribute__((address_space(1))) const char g_char;
+  auto uniform64 = [](uint64_t x) __attribute__((always_inline)) -> uint64_t {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)x);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(x >> 32));
+    return ((uint64_t)hi << 32) | lo;
+  };
+  // pins a uniform address in a scalar register pair, so that the load keeps
+  // the form "scalar base + 32-bit lane offset" (the optimiser would otherwise
+  // fold the lane offset into a 64-bit vector address per load)
+  auto scalar_ptr = [](uint64_t a) __attribute__((always_inline)) -> g_char* {
+    uint32_t lo = (uint32_t)a, hi = (uint32_t)(a >> 32);
+    asm volatile("" : "+s"(lo), "+s"(hi));
+    return (g_char*)(((uint64_t)hi << 32) | lo);
+  };
+  const uint32_t k_step = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)((64 / G::NCH) * p.k_ss * 2));
+  const uint32_t v_step = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)((64 / G::NCH) * p.v_ss * 2));
+  const uint32_t k_lane = (uint32_t)((lane / G::NCH) * p.k_ss * 2 + (lane % G::NCH) * 16);
+  const uint32_t v_lane = (uint32_t)((lane / G::NCH) * p.v_ss * 2 + (lane % G::NCH) * 16);
+  // shift: page_shift() of the tile (0 unless paged)
+  const uint32_t k_rowb = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(p.k_ss * 2));
+  const uint32_t v_rowb = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(p.v_ss * 2));
+  // regs[i] <- chunk (lane + 64 i) of the tile at `tile` (uniform address of
+  // its first row); rows beyond row_max re-read row row_max (the last token:
+  // same tile, hence same page)
+  auto load_tile = [&](i32x4 (&regs)[LOADS], uint64_t tile, int row_max, uint32_t rowb, uint32_t step,
+                       uint32_t lane_off) __attribute__((always_inline)) {
+    if (kUniformRows && row_max >= kDecTile - 1) {
+#pragma unroll
+      for (int i = 0; i < LOADS; ++i)
+        regs[i] = __builtin_nontemporal_load((g_i32x4*)(scalar_ptr(tile + (uint64_t)i * step) + lane_off));
+      return;
+    }
+    g_char* base = scalar_ptr(tile);
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       const int idx = lane + i * 64;
       if (NCHUNK % 64 == 0 || idx < NCHUNK) {
         const int row = idx / G::NCH, ch = idx % G::NCH;
-        // rows past the end re-read the last token (same tile, hence same page)
-        const int64_t kr = min(tb + row, len - 1);
-        kreg[i] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(kp + kshift + kr * p.k_ss + ch * 8));
-        vreg[i] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(vp + vshift + kr * p.v_ss + ch * 8));
+        const uint32_t off = (uint32_t)min(row, row_max) * rowb + ch * 16;
+        regs[i] = __builtin_nontemporal_load((g_i32x4*)(base + off));
       }
     }
   };
-  auto lstore = [&]() {
+  auto gload = [&](int base, int64_t kshift, int64_t vshift) __attribute__((always_inline)) {
+    const int tb = addr_base(base);
+    load_tile(kreg, uniform64((uint64_t)(uintptr_t)(kp + kshift + (int64_t)tb * p.k_ss)), len - 1 - tb, k_rowb, k_step,
+              k_lane);
+    load_tile(vreg, uniform64((uint64_t)(uintptr_t)(vp + vshift + (int64_t)tb * p.v_ss)), len - 1 - tb, v_rowb, v_step,
+              v_lane);
+  };
+  auto lstore = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       const int idx = lane + i * 64;
@@ -148,13 +192,12 @@ decode_splitkv_kernel(const DecodeParams p) {
   const int wl = p.win_local, wg = p.win_global;
   // tile bases and page look-ups run one tile ahead of the loads that use
   // them, which run one tile ahead of the compute
+  auto shift_k = [&](int base) -> int64_t { return page_shift(addr_base(base), p.k_sb, p.k_ss); };
+  auto shift_v = [&](int base) -> int64_t { return page_shift(addr_base(base), p.v_sb, p.v_ss); };
   int base_cur = tile_base(0);
-  {
-    const int tb = addr_base(base_cur);
-    gload(base_cur, page_shift(tb, p.k_sb, p.k_ss), page_shift(tb, p.v_sb, p.v_ss));
-  }
+  gload(base_cur, shift_k(base_cur), shift_v(base_cur));
   int base_nxt = n_tiles > 1 ? tile_base(1) : 0;
-  int64_t ks_nxt = page_shift(addr_base(base_nxt), p.k_sb, p.k_ss), vs_nxt = page_shift(addr_base(base_nxt), p.v_sb, p.v_ss);
+  int64_t ks_nxt = shift_k(base_nxt), vs_nxt = shift_v(base_nxt);
   lstore();
   for (int it = 0; it < n_tiles; ++it) {
     const int base = base_cur;
@@ -163,8 +206,8 @@ decode_splitkv_kernel(const DecodeParams p) {
     base_cur = base_nxt;
     if (it + 2 < n_tiles) {
       base_nxt = tile_base(it + 2);
-      ks_nxt = page_shift(addr_base(base_nxt), p.k_sb, p.k_ss);
-      vs_nxt = page_shift(addr_base(base_nxt), p.v_sb, p.v_ss);
+      ks_nxt = shift_k(base_nxt);
+      vs_nxt = shift_v(base_nxt);
     }
     bool need_mask = base + kDecTile > len || base < 0;
     if (wl >= 0) need_mask = need_mask || !((base + kDecTile - 1 < wg) || (base >= len - wl));
