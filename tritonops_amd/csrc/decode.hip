@@ -5,15 +5,20 @@
 // of flash_attn_triton/flash_attn_decoding.py:9-122,:126-210 and their sparse
 // twins in flash_attn_triton/flash_attn_decoding_sparse.py:10-127,:131-219.
 //
-// Pass 1: one wavefront (= one workgroup) per (chunk, kv-head, sequence).  The
-// G = hq/hkv query heads that share the kv-head sit in the first G of the 32
+// Pass 1: a work item is a (chunk, kv-head, sequence) triple and is handled
+// by one wavefront (= one workgroup).  The block-list form launches one
+// wavefront per item; the dense form launches one resident round of wavefronts
+// (8 per CU) and deals the live chunks of a ragged batch to them round-robin.
+// The G = hq/hkv query heads that share the kv-head sit in the first G of the 32
 // query columns of the same S^T = K.Q^T / O^T = V^T.P^T MFMA pipeline the
 // prefill kernel uses, so each K/V byte is fetched once for the whole group
 // (the reference launches one program per q-head and re-reads KV G times,
 // flash_attn_decoding.py:42-45,264-268) and the dot products cost no VALU
 // work.  KV streams global -> registers -> wave-private LDS in 32-key tiles
-// with fully coalesced 16-byte loads; no barriers are needed because a single
-// wave's LDS operations execute in order.  Partials are fp32 (the reference
+// with fully coalesced 16-byte loads (non-temporal: every byte is used once);
+// as soon as a tile has arrived, each register is written to LDS and refilled
+// with its part of the tile after next.  No barriers are needed because a
+// single wave's LDS operations execute in order.  Partials are fp32 (the reference
 // rounds them to the input dtype, :249-251).
 // Pass 2: per (sequence, q-head) merge  o = sum_c o_c 2^(lse_c - lse).
 #include "kernels.h"
@@ -24,22 +29,20 @@ namespace {
 
 constexpr int kDecTile = 32;
 
+// One work item: chunk `split` of (sequence b, kv-head kvh).
 template <typename T, int D>
-__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2)))
-decode_splitkv_kernel(const DecodeParams p) {
+__device__ __forceinline__ void decode_item(const DecodeParams& p, unsigned char* smem, const int split, const int kvh,
+                                            const int b) {
   using G = RowGeom<D>;
   using F = PaddedFrags<D>;
   constexpr int KTILEB = kDecTile * F::KROWB;
-  constexpr int VTILEB = kDecTile * F::VROWB;
   constexpr int NCHUNK = kDecTile * G::NCH;
   constexpr int LOADS = (NCHUNK + 63) / 64;
 
-  __shared__ __attribute__((aligned(16))) unsigned char smem[KTILEB + VTILEB];
   unsigned char* sK = smem;
   unsigned char* sV = smem + KTILEB;
 
   const int lane = threadIdx.x;
-  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
   const int len = p.seq_lens ? p.seq_lens[b] : p.cu[b + 1] - p.cu[b];
   const int gqa = p.hq / p.hkv;
   const bool sparse = p.block_idx != nullptr;
@@ -145,69 +148,75 @@ decode_splitkv_kernel(const DecodeParams p) {
   const uint32_t v_step = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)((64 / G::NCH) * p.v_ss * 2));
   const uint32_t k_lane = (uint32_t)((lane / G::NCH) * p.k_ss * 2 + (lane % G::NCH) * 16);
   const uint32_t v_lane = (uint32_t)((lane / G::NCH) * p.v_ss * 2 + (lane % G::NCH) * 16);
-  // shift: page_shift() of the tile (0 unless paged)
   const uint32_t k_rowb = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(p.k_ss * 2));
   const uint32_t v_rowb = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(p.v_ss * 2));
-  // regs[i] <- chunk (lane + 64 i) of the tile at `tile` (uniform address of
-  // its first row); rows beyond row_max re-read row row_max (the last token:
-  // same tile, hence same page)
-  auto load_tile = [&](i32x4 (&regs)[LOADS], uint64_t tile, int row_max, uint32_t rowb, uint32_t step,
-                       uint32_t lane_off) __attribute__((always_inline)) {
+  // reg <- chunk (lane + 64 i) of the tile at `tile` (uniform address of its
+  // first row); rows beyond row_max re-read row row_max (the last token: same
+  // tile, hence same page)
+  auto load_one = [&](i32x4& reg, int i, uint64_t tile, int row_max, uint32_t rowb, uint32_t step,
+                      uint32_t lane_off) __attribute__((always_inline)) {
+    const int idx = lane + i * 64;
+    if (NCHUNK % 64 != 0 && idx >= NCHUNK) return;
     if (kUniformRows && row_max >= kDecTile - 1) {
-#pragma unroll
-      for (int i = 0; i < LOADS; ++i)
-        regs[i] = __builtin_nontemporal_load((g_i32x4*)(scalar_ptr(tile + (uint64_t)i * step) + lane_off));
-      return;
-    }
-    g_char* base = scalar_ptr(tile);
-#pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-      const int idx = lane + i * 64;
-      if (NCHUNK % 64 == 0 || idx < NCHUNK) {
-        const int row = idx / G::NCH, ch = idx % G::NCH;
-        const uint32_t off = (uint32_t)min(row, row_max) * rowb + ch * 16;
-        regs[i] = __builtin_nontemporal_load((g_i32x4*)(base + off));
-      }
+      reg = __builtin_nontemporal_load((g_i32x4*)(scalar_ptr(tile + (uint64_t)i * step) + lane_off));
+    } else {
+      const int row = idx / G::NCH, ch = idx % G::NCH;
+      const uint32_t off = (uint32_t)min(row, row_max) * rowb + ch * 16;
+      reg = __builtin_nontemporal_load((g_i32x4*)(scalar_ptr(tile) + off));
     }
   };
-  auto gload = [&](int base, int64_t kshift, int64_t vshift) __attribute__((always_inline)) {
+  auto store_one = [&](int i) __attribute__((always_inline)) {
+    const int idx = lane + i * 64;
+    if (NCHUNK % 64 != 0 && idx >= NCHUNK) return;
+    const int row = idx / G::NCH, ch = idx % G::NCH;
+    F::store_k(sK, row, ch, kreg[i]);
+    F::store_v(sV, row, ch, vreg[i]);
+  };
+  // where a tile comes from: uniform addresses of its first K / V row and the
+  // last row that may be read
+  struct TileSrc {
+    uint64_t k, v;
+    int row_max;
+  };
+  auto tile_src = [&](int base) __attribute__((always_inline)) -> TileSrc {
     const int tb = addr_base(base);
-    load_tile(kreg, uniform64((uint64_t)(uintptr_t)(kp + kshift + (int64_t)tb * p.k_ss)), len - 1 - tb, k_rowb, k_step,
-              k_lane);
-    load_tile(vreg, uniform64((uint64_t)(uintptr_t)(vp + vshift + (int64_t)tb * p.v_ss)), len - 1 - tb, v_rowb, v_step,
-              v_lane);
+    TileSrc t;
+    t.k = uniform64((uint64_t)(uintptr_t)(kp + page_shift(tb, p.k_sb, p.k_ss) + (int64_t)tb * p.k_ss));
+    t.v = uniform64((uint64_t)(uintptr_t)(vp + page_shift(tb, p.v_sb, p.v_ss) + (int64_t)tb * p.v_ss));
+    t.row_max = len - 1 - tb;
+    return t;
   };
-  auto lstore = [&]() __attribute__((always_inline)) {
-#pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-      const int idx = lane + i * 64;
-      if (NCHUNK % 64 == 0 || idx < NCHUNK) {
-        const int row = idx / G::NCH, ch = idx % G::NCH;
-        F::store_k(sK, row, ch, kreg[i]);
-        F::store_v(sV, row, ch, vreg[i]);
-      }
-    }
+  auto load_pair = [&](int i, const TileSrc& t) __attribute__((always_inline)) {
+    load_one(kreg[i], i, t.k, t.row_max, k_rowb, k_step, k_lane);
+    load_one(vreg[i], i, t.v, t.row_max, v_rowb, v_step, v_lane);
   };
 
   const int wl = p.win_local, wg = p.win_global;
-  // tile bases and page look-ups run one tile ahead of the loads that use
-  // them, which run one tile ahead of the compute
-  auto shift_k = [&](int base) -> int64_t { return page_shift(addr_base(base), p.k_sb, p.k_ss); };
-  auto shift_v = [&](int base) -> int64_t { return page_shift(addr_base(base), p.v_sb, p.v_ss); };
+  // Tile t is worked on from LDS while tile t + 1 is in flight into the
+  // registers.  When it has arrived, every register is written to LDS and
+  // refilled at once with its part of tile t + 2, so that the next loads leave
+  // as early as possible; the address of tile t + 2 (block list and page
+  // look-ups) is prepared before tile t is worked on.
   int base_cur = tile_base(0);
-  gload(base_cur, shift_k(base_cur), shift_v(base_cur));
+  {
+    const TileSrc t0 = tile_src(base_cur);
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) load_pair(i, t0);
+  }
   int base_nxt = n_tiles > 1 ? tile_base(1) : 0;
-  int64_t ks_nxt = shift_k(base_nxt), vs_nxt = shift_v(base_nxt);
-  lstore();
+  TileSrc src = tile_src(base_nxt);  // tile 1, then the tile two ahead of the compute
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    store_one(i);
+    if (n_tiles > 1) load_pair(i, src);
+  }
   for (int it = 0; it < n_tiles; ++it) {
     const int base = base_cur;
-    const bool more = it + 1 < n_tiles;
-    if (more) gload(base_nxt, ks_nxt, vs_nxt);
     base_cur = base_nxt;
-    if (it + 2 < n_tiles) {
+    const bool refill = it + 2 < n_tiles;
+    if (refill) {
       base_nxt = tile_base(it + 2);
-      ks_nxt = shift_k(base_nxt);
-      vs_nxt = shift_v(base_nxt);
+      src = tile_src(base_nxt);
     }
     bool need_mask = base + kDecTile > len || base < 0;
     if (wl >= 0) need_mask = need_mask || !((base + kDecTile - 1 < wg) || (base >= len - wl));
@@ -218,7 +227,13 @@ decode_splitkv_kernel(const DecodeParams p) {
       return ok;
     };
     compute_tile<T, D, 1>(sK, sV, lc, Qf, O, m, l, p.scale, need_mask, allowed);
-    if (more) lstore();
+    if (it + 1 < n_tiles) {
+#pragma unroll
+      for (int i = 0; i < LOADS; ++i) {
+        store_one(i);
+        if (refill) load_pair(i, src);
+      }
+    }
   }
 
   const float l_tot = sum_with_other_half(l);
@@ -236,6 +251,65 @@ decode_splitkv_kernel(const DecodeParams p) {
                     O[db][4 * g + 3] * inv};
         *reinterpret_cast<float4*>(po + 32 * db + 8 * g + 4 * lc.lh) = w;
       }
+  }
+}
+
+// Block-list form: one wavefront per (chunk, kv-head, sequence), grid
+// (n_splits, hkv, batch).  Dense form: the live chunks of all sequences (a
+// sequence of length L has ceil(L / split_tokens) of them) are numbered
+// consecutively and dealt round-robin to gridDim.x wavefronts, one resident
+// round of the chip, so that ragged batches leave no tail of half-empty rounds:
+// every wavefront gets the same number of chunks, give or take one.
+template <typename T, int D>
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2)))
+decode_splitkv_kernel(const DecodeParams p) {
+  using F = PaddedFrags<D>;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[kDecTile * (F::KROWB + F::VROWB)];
+  if (p.block_idx != nullptr) {
+    decode_item<T, D>(p, smem, blockIdx.x, blockIdx.y, blockIdx.z);
+    return;
+  }
+  const int lane = threadIdx.x;
+  auto chunks_of = [&](int b) -> int {
+    if (b >= p.batch) return 0;
+    const int len = p.seq_lens ? p.seq_lens[b] : p.cu[b + 1] - p.cu[b];
+    return max(0, min((len + p.split_tokens - 1) / p.split_tokens, p.n_splits));
+  };
+  // chunks of all sequences (wave-wide sum, 64 sequences per step)
+  int total = 0;
+  for (int b0 = 0; b0 < p.batch; b0 += 64) {
+    int c = chunks_of(b0 + lane);
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) c += __shfl_xor(c, m, 64);
+    total += c;
+  }
+  total = __builtin_amdgcn_readfirstlane(total);
+  const long long items = (long long)total * p.hkv;
+  for (long long g = blockIdx.x; g < items; g += gridDim.x) {
+    const int t = (int)(g / p.hkv), kvh = (int)(g % p.hkv);
+    // sequence that owns live chunk t: inclusive scan over the chunk counts
+    int b = 0, first = 0;
+    for (int b0 = 0, seen = 0; b0 < p.batch; b0 += 64) {
+      const int c = chunks_of(b0 + lane);
+      int incl = c;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += up;
+      }
+      const int before = seen + incl - c;  // live chunks ahead of this lane's sequence
+      const unsigned long long hit = __builtin_amdgcn_ballot_w64(c > 0 && t >= before && t < before + c);
+      if (hit) {
+        const int src = __builtin_ctzll(hit);
+        b = b0 + src;
+        first = __shfl(before, src, 64);
+        break;
+      }
+      seen += __shfl(incl, 63, 64);
+    }
+    b = __builtin_amdgcn_readfirstlane(b);
+    first = __builtin_amdgcn_readfirstlane(first);
+    decode_item<T, D>(p, smem, t - first, kvh, b);
   }
 }
 
@@ -275,9 +349,23 @@ decode_merge_kernel(const DecodeParams p, int D) {
   if (d == 0 && p.lse) p.lse[(int64_t)b * p.hq + h] = den > 0.f ? M + fast_log2(den) : -INFINITY;
 }
 
+int decode_cu_count() {
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+    n = 256;
+  return n;
+}
+
 template <typename T, int D>
 int launch_split(const DecodeParams& p, hipStream_t s) {
   dim3 grid(p.n_splits, p.hkv, p.batch);
+  if (p.block_idx == nullptr) {
+    // dense: one resident round (8 wavefronts per CU), fewer when there are fewer chunks
+    const long long slots = (long long)p.n_splits * p.hkv * p.batch;
+    const long long resident = 8LL * decode_cu_count();
+    grid = dim3((unsigned)(slots < resident ? slots : resident), 1, 1);
+  }
   hipLaunchKernelGGL((decode_splitkv_kernel<T, D>), grid, dim3(64), 0, s, p);
   return (int)hipGetLastError();
 }
