@@ -89,12 +89,14 @@ struct UniFrags {
 
 extern __shared__ __attribute__((aligned(1024))) unsigned char smem_bwd[];
 
+constexpr int kBwdStages = 3;  // streamed tile pairs resident in LDS (4 measured the same)
+
 template <typename T, int D, int MODE>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2)))
 bwd_kernel(const BwdParams p) {
   using G = RowGeom<D>;
   using F = UniFrags<D>;
-  constexpr int NW = 8, BM = 32 * NW, TN = 64, NS = 3;
+  constexpr int NW = 8, BM = 32 * NW, TN = 64, NS = kBwdStages;
   constexpr int TILEB = TN * F::ROWB;             // one streamed tile
   constexpr int STAGEB = 2 * TILEB + 1024;        // tile 0, tile 1, lse[64] and delta[64] (fp32)
   constexpr int RPI = 1024 / F::ROWB;             // tile rows per direct-to-LDS instruction
@@ -382,9 +384,12 @@ bwd_kernel(const BwdParams p) {
     const bool refill = u + NS - 1 < n_stream;
     if (refill) issue(u + NS - 1, ic<(ST + NS - 1) % NS>{});
     compute(u, stage_c);
-    // the next tile must have landed (this wave's loads retire in order: at
-    // most the youngest tile's may still fly) and everyone is done with this one
-    if (refill)
+    // the next tile must have landed (this wave's loads retire in order: only
+    // the tiles requested after it may still fly) and everyone is done with this one
+    const int younger = min(n_stream - 1, u + NS - 1) - (u + 1);
+    if (younger >= 2)
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * IPT));
+    else if (younger == 1)
       __builtin_amdgcn_s_waitcnt(waitcnt_vm(IPT));
     else
       __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
@@ -393,6 +398,7 @@ bwd_kernel(const BwdParams p) {
 
   if (n_stream > 0) issue(0, ic<0>{});
   if (n_stream > 1) issue(1, ic<1>{});
+  if (NS > 3 && n_stream > 2) issue(2, ic<2 % NS>{});
   // resident operands and tile 0 are needed now; the full wait also tells the
   // compiler that no register load is pending inside the loop
   __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
@@ -403,6 +409,10 @@ bwd_kernel(const BwdParams p) {
     step(ic<1>{}, u + 1);
     if (u + 2 >= n_stream) break;
     step(ic<2>{}, u + 2);
+    if (NS > 3) {
+      if (u + 3 >= n_stream) break;
+      step(ic<3 % NS>{}, u + 3);
+    }
   }
   __syncthreads();
 
@@ -478,7 +488,7 @@ __global__ void __launch_bounds__(256) bwd_delta_kernel(const BwdParams p, int h
 
 template <typename T, int D, int MODE>
 int launch_mode(const BwdParams& p, hipStream_t s) {
-  constexpr size_t lds = 3 * (2 * 64 * 256 + 1024);
+  constexpr size_t lds = kBwdStages * (2 * 64 * 256 + 1024);
   static_assert(lds >= 8 * 32 * (D * 2 + 16), "epilogue staging must fit the tile ring");
   auto kern = bwd_kernel<T, D, MODE>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
