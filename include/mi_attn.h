@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define MI_ATTN_ABI_VERSION 3
+#define MI_ATTN_ABI_VERSION 4
 
 /* KV tile edge (tokens) of the prefill kernels and block edge of the block
  * sparse layouts; fixed at build time. */
@@ -364,6 +364,29 @@ typedef struct mi_xent_args {
 size_t mi_xent_fwd_workspace_bytes(const mi_xent_args *args);
 int mi_xent_fwd(const mi_xent_args *args, void *stream);
 
+/* Backward, first step: dlogits[t,n] = dloss[t] (exp(logits[t,n] - lse[t]) -
+ * [n == y[t]]) for a block of tokens, computed by the forward's GEMM kernel
+ * with this epilogue on the fp32 accumulators and written once, in the dtype
+ * of x.  Replaces `xw_partial = torch.mm(x_partial, w^T)` plus
+ * cross_entropy_fused_bwd_kernel (cross_entropy.py:374, :185-266), which round
+ * the logits to the storage dtype before the exponential.  The two gradient
+ * GEMMs (grad_x = dlogits w, grad_w = dlogits^T x, :407-415) stay with the
+ * caller's BLAS.  x / w / y as for mi_xent_fwd; no workspace. */
+typedef struct mi_xent_bwd_args {
+  uint32_t struct_size;
+  int32_t dtype;                 /* of x, w and dlogits                        */
+  int32_t tokens, dim, vocab;
+  int32_t labels_i64;
+  const void *x, *w;             /* device                                     */
+  const void *y;                 /* [tokens] labels                            */
+  int64_t x_stride, w_stride;    /* row strides, elements                      */
+  const float *lse, *dloss;      /* [tokens] fp32                              */
+  void *dlogits;                 /* [tokens, vocab], row stride ld (elements)  */
+  int64_t ld;
+} mi_xent_bwd_args;
+
+int mi_xent_bwd_dlogits(const mi_xent_bwd_args *args, void *stream);
+
 /* In place over a block of logits [rows, vocab] (row stride ld, elements):
  * logits[t,n] <- dloss[t] (exp(logits[t,n] - lse[t]) - [n == y[t]]), the
  * operand of the two gradient GEMMs (cross_entropy.py:255-266, :369-415). */
@@ -399,7 +422,7 @@ int mi_attn_bwd_validate(const mi_attn_bwd_args *args);
  * kind: 0 = mi_attn_fwd, 1 = mi_attn_fwd_blocksparse, 2 = mi_decode,
  *       3 = mi_decode_splitkv, 4 = mi_decode_merge, 5 = mi_attn_bwd,
  *       6 = mi_rmsnorm_fwd, 7 = mi_rmsnorm_bwd, 8 = mi_xent_fwd,
- *       9 = mi_xent_dlogits.
+ *       9 = mi_xent_dlogits, 10 = mi_xent_bwd_dlogits.
  * Returns MI_OK and writes milliseconds to *ms_per_launch. */
 int mi_time_launches(int kind, const void *args, void *stream, int warmup,
                      int iters, float *ms_per_launch);

@@ -27,19 +27,20 @@ def test_every_declared_symbol_is_exported(lib):
     assert declared == set(_lib.EXPORTS), "ctypes table and header disagree: %s" % (declared ^ set(_lib.EXPORTS))
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.mi_abi_version() == _lib.MI_ATTN_ABI_VERSION == 3
+    assert lib.mi_abi_version() == _lib.MI_ATTN_ABI_VERSION == 4
 
 
 def test_struct_layout_matches_the_c_compiler(tmp_path):
     src = tmp_path / "sz.c"
-    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "mi_attn.h"\nint main(){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\\n",'
+    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "mi_attn.h"\nint main(){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\\n",'
                    "sizeof(mi_attn_fwd_args),sizeof(mi_attn_sparse_args),sizeof(mi_decode_args),"
                    "offsetof(mi_attn_fwd_args,scale_log2),offsetof(mi_attn_sparse_args,scale_log2),"
                    "offsetof(mi_decode_args,page_table),"
                    "sizeof(mi_attn_bwd_args),offsetof(mi_attn_bwd_args,workspace),"
                    "sizeof(mi_rmsnorm_args),offsetof(mi_rmsnorm_args,eps),"
                    "sizeof(mi_xent_args),offsetof(mi_xent_args,workspace),"
-                   "sizeof(mi_xent_grad_args),offsetof(mi_xent_grad_args,y));return 0;}\n")
+                   "sizeof(mi_xent_grad_args),offsetof(mi_xent_grad_args,y),"
+                   "sizeof(mi_xent_bwd_args),offsetof(mi_xent_bwd_args,ld));return 0;}\n")
     exe = tmp_path / "sz"
     subprocess.check_call(["gcc", "-std=c99", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
     got = [int(x) for x in subprocess.check_output([str(exe)]).split()]
@@ -49,7 +50,8 @@ def test_struct_layout_matches_the_c_compiler(tmp_path):
             C.sizeof(_lib.AttnBwdArgs), _lib.AttnBwdArgs.workspace.offset,
             C.sizeof(_lib.RmsNormArgs), _lib.RmsNormArgs.eps.offset,
             C.sizeof(_lib.XentArgs), _lib.XentArgs.workspace.offset,
-            C.sizeof(_lib.XentGradArgs), _lib.XentGradArgs.y.offset]
+            C.sizeof(_lib.XentGradArgs), _lib.XentGradArgs.y.offset,
+            C.sizeof(_lib.XentBwdArgs), _lib.XentBwdArgs.ld.offset]
     assert got == want
 
 
@@ -281,6 +283,20 @@ def test_fused_cross_entropy_validation(lib):
     a.tokens, a.vocab = 100, 1000
     assert lib.mi_xent_fwd_workspace_bytes(C.byref(a)) == 100 * 4 * 2 * 4
 
+    b = _lib.XentBwdArgs()
+    b.struct_size = C.sizeof(b)
+    b.dtype, b.tokens, b.dim, b.vocab, b.labels_i64 = 0, 512, 1024, 32000, 0
+    b.x = b.w = b.y = b.lse = b.dloss = b.dlogits = 0x1000
+    b.x_stride = b.w_stride = 1024
+    b.ld = 31999
+    assert lib.mi_status_name(lib.mi_xent_bwd_dlogits(C.byref(b), None)).decode() == "MI_ERR_STRIDE"
+    b.ld, b.dim = 32000, 1000
+    assert lib.mi_status_name(lib.mi_xent_bwd_dlogits(C.byref(b), None)).decode() == "MI_ERR_SHAPE"
+    b.dim, b.dloss = 1024, None
+    assert lib.mi_status_name(lib.mi_xent_bwd_dlogits(C.byref(b), None)).decode() == "MI_ERR_NULL_POINTER"
+    b.tokens = 0
+    assert lib.mi_xent_bwd_dlogits(C.byref(b), None) == 0
+
     g = _lib.XentGradArgs()
     g.struct_size = C.sizeof(g)
     g.dtype, g.vocab, g.labels_i64, g.rows, g.ld = 0, 1000, 1, 16, 900
@@ -311,7 +327,7 @@ def test_time_launches_rejects_bad_arguments(lib):
     ms = C.c_float()
     assert lib.mi_time_launches(0, None, None, 0, 1, C.byref(ms)) == -1
     a = _good_fwd()
-    assert lib.mi_time_launches(10, C.cast(C.byref(a), C.c_void_p), None, 0, 1, C.byref(ms)) == -6
+    assert lib.mi_time_launches(11, C.cast(C.byref(a), C.c_void_p), None, 0, 1, C.byref(ms)) == -6
     a.head_dim = 5
     assert lib.mi_time_launches(0, C.cast(C.byref(a), C.c_void_p), None, 1, 1, C.byref(ms)) == -4
 

@@ -164,3 +164,24 @@ def test_full_size_is_invariant_to_the_launch_shape():
     logits = x[:64].float() @ w.float().t()
     want = torch.logsumexp(logits, -1) - logits.gather(-1, y[:64].view(-1, 1)).squeeze(-1)
     assert (loss[:64] - want).abs().max().item() <= 2e-3
+
+
+@pytest.mark.parametrize("T,D,N", [(300, 256, 1000), (257, 128, 4096 + 37), (64, 384, 263)])
+def test_dlogits_from_the_gemm_kernel(T, D, N):
+    """The gradient epilogue against float64 math, with logits large enough
+    (|logit| up to ~60) that rounding them to bf16 first would be visible:
+    partial token / vocabulary tiles, N not a multiple of 8 (element-wise stores)."""
+    import tritonops_amd as ta
+
+    x = _rand((T, D), 21, torch.bfloat16)
+    w = _rand((N, D), 22, torch.bfloat16, scale=1.2)
+    y = _labels(T, N, 23)
+    go = _rand((T,), 24)
+    logits = x.double() @ w.double().t()
+    lse = torch.logsumexp(logits, -1)
+    want = go.double().view(-1, 1) * (torch.exp(logits - lse.view(-1, 1)) - torch.nn.functional.one_hot(y, N).double())
+    got = ta.cross_entropy_dlogits(x.cuda(), w.cuda(), y.cuda(), lse.float().cuda(), go.cuda())
+    assert got.shape == (T, N) and got.dtype == torch.bfloat16
+    assert (got.cpu().double() - want).abs().max() <= 1e-2 * max(1.0, want.abs().max().item())
+    # rows sum to zero up to the rounding of the stored values
+    assert got.float().sum(-1).abs().max().item() <= 0.1 * go.abs().max().item()

@@ -13,6 +13,7 @@ from .ops import (  # noqa: F401
 from .rms import RMSNormTriton, RMSNormTritonFunction, rmsnorm_bwd, rmsnorm_fwd  # noqa: F401
 from .xent import (  # noqa: F401
     CrossEntropyFusedFunction,
+    cross_entropy_dlogits,
     cross_entropy_dlogits_,
     cross_entropy_fused_bwd,
     cross_entropy_fused_fwd,

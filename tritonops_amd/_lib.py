@@ -9,7 +9,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmi_attn.so")
 
-MI_ATTN_ABI_VERSION = 3
+MI_ATTN_ABI_VERSION = 4
 MI_KV_BATCHED, MI_KV_PACKED, MI_KV_PAGED = 0, 1, 2
 MI_ATTN_BLOCK = 64
 MI_DTYPE_F32 = 2
@@ -108,6 +108,17 @@ class XentArgs(C.Structure):
     ]
 
 
+class XentBwdArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", _u32), ("dtype", _i32),
+        ("tokens", _i32), ("dim", _i32), ("vocab", _i32), ("labels_i64", _i32),
+        ("x", _vp), ("w", _vp), ("y", _vp),
+        ("x_stride", _i64), ("w_stride", _i64),
+        ("lse", _vp), ("dloss", _vp),
+        ("dlogits", _vp), ("ld", _i64),
+    ]
+
+
 class XentGradArgs(C.Structure):
     _fields_ = [
         ("struct_size", _u32), ("dtype", _i32), ("vocab", _i32), ("labels_i64", _i32),
@@ -153,6 +164,7 @@ EXPORTS = {
     "mi_xent_fwd": (C.c_int, [C.POINTER(XentArgs), _vp]),
     "mi_xent_fwd_workspace_bytes": (_sz, [C.POINTER(XentArgs)]),
     "mi_xent_dlogits": (C.c_int, [C.POINTER(XentGradArgs), _vp]),
+    "mi_xent_bwd_dlogits": (C.c_int, [C.POINTER(XentBwdArgs), _vp]),
     "mi_decode_num_splits": (C.c_int, [C.POINTER(DecodeArgs)]),
     "mi_decode_workspace_bytes": (_sz, [C.POINTER(DecodeArgs)]),
     "mi_decode_choose_split_tokens": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int]),

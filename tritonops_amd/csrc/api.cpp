@@ -269,7 +269,36 @@ int mi_xent_fwd(const mi_xent_args* a, void* stream) {
   p.lse_part = static_cast<float*>(a->workspace);
   p.tgt_part = p.lse_part + (size_t)a->tokens * p.n_split;
   p.lse = a->lse; p.loss = a->loss;
-  return launch_status(mi::launch_xent_fwd(p, a->dtype, static_cast<hipStream_t>(stream)), "mi_xent_fwd");
+  return launch_status(mi::launch_xent_fwd(p, a->dtype, false, static_cast<hipStream_t>(stream)), "mi_xent_fwd");
+}
+
+int mi_xent_bwd_dlogits(const mi_xent_bwd_args* a, void* stream) {
+  if (!a) return fail(MI_ERR_NULL_POINTER, "args is NULL");
+  if (a->struct_size != sizeof(mi_xent_bwd_args))
+    return fail(MI_ERR_STRUCT_SIZE, "mi_xent_bwd_args.struct_size %u != %zu", a->struct_size, sizeof(mi_xent_bwd_args));
+  if (a->dtype != MI_DTYPE_BF16 && a->dtype != MI_DTYPE_F16) return fail(MI_ERR_DTYPE, "dtype %d is not bf16 / f16", a->dtype);
+  if (a->tokens < 0 || a->dim <= 0 || a->vocab <= 0)
+    return fail(MI_ERR_SHAPE, "tokens %d must be >= 0, dim %d and vocab %d positive", a->tokens, a->dim, a->vocab);
+  if (a->dim % 128) return fail(MI_ERR_SHAPE, "dim %d must be a multiple of 128 (pad with zero columns)", a->dim);
+  if (a->labels_i64 != 0 && a->labels_i64 != 1) return fail(MI_ERR_SHAPE, "labels_i64 must be 0 or 1");
+  if (a->tokens == 0) return MI_OK;
+  if (!a->x || !a->w || !a->y || !a->lse || !a->dloss || !a->dlogits)
+    return fail(MI_ERR_NULL_POINTER, "x, w, y, lse, dloss and dlogits must be non-NULL");
+  if (!aligned16(a->x) || !aligned16(a->w)) return fail(MI_ERR_ALIGNMENT, "x and w must be 16-byte aligned");
+  if (a->x_stride < a->dim || a->w_stride < a->dim || a->x_stride % 8 || a->w_stride % 8)
+    return fail(MI_ERR_STRIDE, "row strides must be >= dim and multiples of 8 elements");
+  if (a->x_stride > (1 << 22) || a->w_stride > (1 << 22)) return fail(MI_ERR_STRIDE, "row stride beyond 2^22 elements");
+  if (a->ld < a->vocab) return fail(MI_ERR_STRIDE, "ld %lld < vocab", (long long)a->ld);
+  mi::XentParams p;
+  std::memset(&p, 0, sizeof(p));
+  p.x = a->x; p.w = a->w; p.y = a->y; p.y_is_i64 = a->labels_i64;
+  p.x_st = a->x_stride; p.w_st = a->w_stride;
+  p.T = a->tokens; p.D = a->dim; p.N = a->vocab;
+  p.n_split = mi::xent_choose_splits(a->tokens, a->vocab, 256);
+  p.lse = const_cast<float*>(a->lse); p.dloss = a->dloss;
+  p.dlogits = a->dlogits; p.dl_ld = a->ld;
+  p.dl_vec = aligned16(a->dlogits) && a->ld % 8 == 0;
+  return launch_status(mi::launch_xent_fwd(p, a->dtype, true, static_cast<hipStream_t>(stream)), "mi_xent_bwd_dlogits");
 }
 
 int mi_xent_dlogits(const mi_xent_grad_args* a, void* stream) {
@@ -524,7 +553,7 @@ int mi_decode(const mi_decode_args* a, void* stream) {
 
 int mi_time_launches(int kind, const void* args, void* stream, int warmup, int iters, float* ms_per_launch) {
   if (!args || !ms_per_launch) return fail(MI_ERR_NULL_POINTER, "args / ms_per_launch is NULL");
-  if (iters <= 0 || warmup < 0 || kind < 0 || kind > 9) return fail(MI_ERR_SHAPE, "bad kind / warmup / iters");
+  if (iters <= 0 || warmup < 0 || kind < 0 || kind > 10) return fail(MI_ERR_SHAPE, "bad kind / warmup / iters");
   auto once = [&]() -> int {
     switch (kind) {
       case 0: return mi_attn_fwd(static_cast<const mi_attn_fwd_args*>(args), stream);
@@ -536,6 +565,7 @@ int mi_time_launches(int kind, const void* args, void* stream, int warmup, int i
       case 7: return mi_rmsnorm_bwd(static_cast<const mi_rmsnorm_args*>(args), stream);
       case 8: return mi_xent_fwd(static_cast<const mi_xent_args*>(args), stream);
       case 9: return mi_xent_dlogits(static_cast<const mi_xent_grad_args*>(args), stream);
+      case 10: return mi_xent_bwd_dlogits(static_cast<const mi_xent_bwd_args*>(args), stream);
       default: return mi_decode_merge(static_cast<const mi_decode_args*>(args), stream);
     }
   };

@@ -97,7 +97,11 @@ struct XentParams {
   const void* y;       // [T] int32 or int64 labels
   float* lse_part;     // workspace [T][n_split]
   float* tgt_part;     // workspace [T][n_split]
-  float *lse, *loss;   // [T]
+  float *lse, *loss;   // [T]: outputs of the forward; lse is an input of the gradient launch
+  const float* dloss;  // [T], gradient launch
+  void* dlogits;       // [T, N] row stride dl_ld (elements), gradient launch
+  int64_t dl_ld;
+  int32_t dl_vec;      // dlogits rows can be written in 16-byte pieces
   int64_t x_st, w_st;
   int32_t T, D, N;
   int32_t y_is_i64;
@@ -135,7 +139,7 @@ int launch_rms_bwd(const RmsParams& p, int x_dtype, int w_dtype, bool vec, int n
 
 // Fused linear + cross-entropy.  D a multiple of 64, rows 16-byte aligned.
 int xent_choose_splits(long long tokens, int vocab, int num_cus);
-int launch_xent_fwd(const XentParams& p, int dtype, hipStream_t s);       // partials + combine
+int launch_xent_fwd(const XentParams& p, int dtype, bool grad, hipStream_t s);  // forward: partials + combine
 int launch_xent_dlogits(const XentGradParams& p, int dtype, hipStream_t s);
 
 // Query rows per workgroup of the two prefill kernels.

@@ -46,8 +46,14 @@ constexpr int kXLdsBytes = 4 * kXSlabB;     // W stage 0, W stage 1, X stage 0, 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
-template <typename T>
-__global__ void __launch_bounds__(512) xent_fwd_kernel(const XentParams p) {
+// GRAD = false: forward (partial lse and target logit per token and range).
+// GRAD = true: the same product with the epilogue of the backward pass: every
+// tile of logits is turned into dloss[t] (exp(logit - lse[t]) - [n == y[t]])
+// straight from the fp32 accumulators and written to dlogits[t, n] in the
+// storage dtype (the reference rounds the logits to the storage dtype first,
+// cross_entropy.py:374,255-265, which costs accuracy when logits are large).
+template <typename T, bool GRAD>
+__global__ void __launch_bounds__(512) xent_gemm_kernel(const XentParams p) {
   typedef __attribute__((address_space(3))) const i32x4 lds_i32x4;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -193,18 +199,88 @@ __global__ void __launch_bounds__(512) xent_fwd_kernel(const XentParams p) {
 
   // ---- per-token state: tokens t0 + 64 wt + 32 cb + lq
   float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f}, tgt[2] = {0.f, 0.f};
-  long long yv[2];
+  long long yv[2] = {0, 0};
+  if (!GRAD) {
 #pragma unroll
-  for (int cb = 0; cb < 2; ++cb) {
-    const int tok = min(t0 + 64 * wt + 32 * cb + lq, p.T - 1);
-    yv[cb] = p.y_is_i64 ? reinterpret_cast<const long long*>(p.y)[tok]
-                        : (long long)reinterpret_cast<const int*>(p.y)[tok];
+    for (int cb = 0; cb < 2; ++cb) {
+      const int tok = min(t0 + 64 * wt + 32 * cb + lq, p.T - 1);
+      yv[cb] = p.y_is_i64 ? reinterpret_cast<const long long*>(p.y)[tok]
+                          : (long long)reinterpret_cast<const int*>(p.y)[tok];
+    }
   }
 
   // accumulators hold logits of vocabulary rows n0 + 128 wv + 32 rb + 8 (i / 4) + 4 lh + i % 4
   auto finish_tile = [&](int n0) __attribute__((always_inline)) {
     const int nw = n0 + 128 * wv;
-    if (nw < p.N) {
+    if (GRAD) {
+      // The tile is transposed through LDS so that it leaves in 16-byte pieces
+      // of whole 256-byte rows.  The slabs of the step just finished (stage 1:
+      // a tile ends on an odd step) are free until the next step refills them;
+      // each wavefront stages 32 tokens x 128 rows at a time in its own 8 KiB.
+      __syncthreads();  // every wavefront is done reading stage 1
+      typedef __attribute__((address_space(3))) i32x2 lds_w_i32x2;
+      // (opaque copies: the row addresses below must be formed here, not hoisted
+      // out of the main loop into registers that the loop cannot spare)
+      int t0v = t0, ldv = (int)p.dl_ld;
+      asm volatile("" : "+s"(t0v), "+s"(ldv));
+      // per-token inputs are fetched here, once per tile, rather than kept in
+      // registers through the main loop
+      float lse2[2], gl[2];
+      long long yt[2];
+#pragma unroll
+      for (int cb = 0; cb < 2; ++cb) {
+        const int tok = min(t0v + 64 * wt + 32 * cb + lq, p.T - 1);
+        lse2[cb] = p.lse[tok] * kLog2e;
+        gl[cb] = p.dloss[tok];
+        yt[cb] = p.y_is_i64 ? reinterpret_cast<const long long*>(p.y)[tok]
+                            : (long long)reinterpret_cast<const int*>(p.y)[tok];
+      }
+      const uint32_t stg = lds0 + (wave < 4 ? 1 : 3) * kXSlabB + (wave & 3) * 8192;
+#pragma unroll
+      for (int cb = 0; cb < 2; ++cb) {
+        // position of the label inside this wavefront's 128 rows, -1 if elsewhere
+        const long long rel64 = yt[cb] - nw;
+        const int rel = rel64 >= 0 && rel64 < 128 ? (int)rel64 : -1;
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+          for (int g4 = 0; g4 < 4; ++g4) {
+            const int nl = 32 * rb + 8 * g4 + 4 * lh;  // first of this lane's 4 consecutive rows
+            float v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const float pr = exp2f(acc[rb][cb][4 * g4 + j] * kLog2e - lse2[cb]);
+              v[j] = gl[cb] * (pr - (rel == nl + j ? 1.f : 0.f));
+            }
+            const i32x2 pk = {(int)Elem<T>::pack2(v[0], v[1]), (int)Elem<T>::pack2(v[2], v[3])};
+            // 8-byte slot nl / 4 of token row lq, slot pairs swizzled by the row
+            const uint32_t slot = (uint32_t)(nl >> 2) ^ ((lq & 15) << 1);
+            *(lds_w_i32x2*)(uintptr_t)(stg + lq * 256 + slot * 8) = pk;
+            __builtin_amdgcn_sched_barrier(0);  // keeps the register need of this rare block small
+          }
+        // read back: 16 lanes per row
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int r = 4 * i + (lane >> 4), ch = lane & 15;  // token row, 16-byte chunk (8 vocabulary rows)
+          const uint32_t slot = (uint32_t)(2 * ch) ^ ((r & 15) << 1);
+          const i32x4 val = *(lds_i32x4*)(uintptr_t)(stg + r * 256 + slot * 8);
+          const int tok = t0v + 64 * wt + 32 * cb + r;
+          const int n = nw + 8 * ch;
+          if (tok < p.T && n < p.N) {
+            T* dst = reinterpret_cast<T*>(p.dlogits) + (int64_t)tok * ldv + n;
+            if (p.dl_vec && n + 8 <= p.N) {
+              __builtin_nontemporal_store(val, reinterpret_cast<i32x4*>(dst));
+            } else {
+              const T* e = reinterpret_cast<const T*>(&val);
+#pragma unroll
+              for (int j = 0; j < 8; ++j)
+                if (n + j < p.N) dst[j] = e[j];
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    } else if (nw < p.N) {
       if (nw + 128 > p.N) {  // the tile that crosses the end of the vocabulary
 #pragma unroll
         for (int rb = 0; rb < 4; ++rb)
@@ -274,6 +350,7 @@ __global__ void __launch_bounds__(512) xent_fwd_kernel(const XentParams p) {
     }
   }
 
+  if (GRAD) return;
   // ---- lane halves, then the two wavefronts that share tokens
 #pragma unroll
   for (int cb = 0; cb < 2; ++cb) {
@@ -357,27 +434,31 @@ int xent_choose_splits(long long tokens, int vocab, int num_cus) {
   return (int)s;
 }
 
-int launch_xent_fwd(const XentParams& p0, int dtype, hipStream_t s) {
+namespace {
+template <typename T, bool GRAD>
+int launch_gemm(const XentParams& p, unsigned grid, hipStream_t s) {
+  auto kern = xent_gemm_kernel<T, GRAD>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kXLdsBytes);
+  if (e != hipSuccess) return (int)e;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kXLdsBytes, s, p);
+  return (int)hipGetLastError();
+}
+}  // namespace
+
+// grad: the launch writes dlogits instead of the partial lse / target logit
+int launch_xent_fwd(const XentParams& p0, int dtype, bool grad, hipStream_t s) {
   XentParams p = p0;
   p.tiles_t = (p.T + kXTileT - 1) / kXTileT;
   p.block_t = p.tiles_t >= 8 ? 8 : p.tiles_t >= 4 ? 4 : p.tiles_t >= 2 ? 2 : 1;
   const int bs = 32 / p.block_t;
   const long long blocks = (long long)((p.tiles_t + p.block_t - 1) / p.block_t) * ((p.n_split + bs - 1) / bs);
   const unsigned grid = (unsigned)((blocks * 32 + 255) / 256 * 256);
-  hipError_t e;
-  if (dtype == 0) {
-    auto kern = xent_fwd_kernel<__bf16>;
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kXLdsBytes);
-    if (e != hipSuccess) return (int)e;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kXLdsBytes, s, p);
-  } else {
-    auto kern = xent_fwd_kernel<_Float16>;
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kXLdsBytes);
-    if (e != hipSuccess) return (int)e;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kXLdsBytes, s, p);
-  }
-  e = hipGetLastError();
-  if (e != hipSuccess) return (int)e;
+  int rc;
+  if (dtype == 0)
+    rc = grad ? launch_gemm<__bf16, true>(p, grid, s) : launch_gemm<__bf16, false>(p, grid, s);
+  else
+    rc = grad ? launch_gemm<_Float16, true>(p, grid, s) : launch_gemm<_Float16, false>(p, grid, s);
+  if (rc || grad) return rc;
   hipLaunchKernelGGL(xent_combine_kernel, dim3((unsigned)((p.T + 255) / 256)), dim3(256), 0, s, p);
   return (int)hipGetLastError();
 }

@@ -1,9 +1,10 @@
 """Fused linear + cross-entropy with the names of the reference's
 cross_entropy_triton/cross_entropy.py, on the HIP kernels of libmi_attn.so
 (no Triton, no fallback).  The forward never materialises the logits; the
-backward follows the reference's scheme (chunks of rows: logits GEMM,
-element-wise dlogits kernel in place, two gradient GEMMs), with the plain GEMMs
-left to the BLAS library behind torch.mm."""
+backward follows the reference's scheme in blocks of rows, with the logits GEMM
+and the element-wise kernel fused into one launch (the dlogits come straight
+from fp32 accumulators) and the two plain gradient GEMMs left to the BLAS
+library behind torch.mm."""
 import ctypes as C
 
 import torch
@@ -96,21 +97,46 @@ def cross_entropy_dlogits_(logits, lse, dloss, y):
     return logits
 
 
+def cross_entropy_dlogits(x, w, y, lse, dloss):
+    """dlogits [T, N] in x's dtype: dloss[t] (exp(x[t] . w[n] - lse[t]) - [n == y[t]]),
+    computed by the forward's GEMM kernel with the gradient epilogue on its fp32
+    accumulators (replaces the logits GEMM + element-wise kernel of
+    cross_entropy.py:374, :185-266, which round the logits to x's dtype first)."""
+    _require_gpu(x, w, y, lse, dloss)
+    lib = _lib.load()
+    T, N = x.shape[0], w.shape[0]
+    xp, wp = _pad_dim(x), _pad_dim(w)
+    dl = torch.empty((T, N), device=x.device, dtype=x.dtype)
+    a = _lib.XentBwdArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _tag(x)
+    a.tokens, a.dim, a.vocab = T, xp.shape[1], N
+    a.labels_i64 = 1 if y.dtype == torch.int64 else 0
+    a.x, a.w, a.y = _ptr(xp), _ptr(wp), _ptr(y)
+    a.x_stride = xp.stride(0) if T > 1 else xp.shape[1]
+    a.w_stride = wp.stride(0) if N > 1 else wp.shape[1]
+    a.lse, a.dloss = _ptr(lse), _ptr(dloss)
+    a.dlogits, a.ld = _ptr(dl), N
+    _lib.check(lib.mi_xent_bwd_dlogits(C.byref(a), _stream()))
+    return dl
+
+
 def cross_entropy_fused_bwd(grad_o, x, w, y, lse, rows_per_block=None):
     """(grad_x, grad_w) in the dtypes of x and w — backward of
-    CrossEntropyFusedFunction (cross_entropy.py:355-420)."""
+    CrossEntropyFusedFunction (cross_entropy.py:355-420): per block of rows,
+    dlogits from the fused GEMM kernel, then the two gradient GEMMs."""
     _require_gpu(grad_o, x, w, y, lse)
     T = x.shape[0]
     y = _labels(y, T)
     g = grad_o.reshape(-1).to(torch.float32).contiguous()
+    lse = lse.contiguous()
     step = rows_per_block or BWD_ROWS
     grad_x = torch.empty_like(x)
     grad_w = None
     for s in range(0, T, step):
         e = min(s + step, T)
         xc = x[s:e]
-        dl = torch.mm(xc, w.t())
-        cross_entropy_dlogits_(dl, lse[s:e], g[s:e], y[s:e])
+        dl = cross_entropy_dlogits(xc, w, y[s:e], lse[s:e], g[s:e])
         torch.mm(dl, w, out=grad_x[s:e])
         if grad_w is None:
             grad_w = torch.mm(dl.t(), xc)
