@@ -93,3 +93,43 @@ def test_batched_backward_through_the_c_abi(causal):
         _check(dq[b:b + 1], wq, "dq[%d]" % b)
         _check(dk[b:b + 1], wk, "dk[%d]" % b)
         _check(dv[b:b + 1], wv, "dv[%d]" % b)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_flash_attention_is_differentiable(causal):
+    """flash_attention (the README's name for flash_attn_triton.apply) records
+    itself for autograd in both layouts; batched [B,H,S,D] with a custom
+    softmax_scale against autograd through fp32 torch math."""
+    import tritonops_amd as ta
+
+    B, H, S, D = 2, 3, 150, 64
+    q, k, v, do = (randn((B, H, S, D), s) for s in (31, 32, 33, 34))
+    scale = 0.2
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o, lse = ta.flash_attention(qg, kg, vg, causal=causal, softmax_scale=scale, return_lse=True)
+    assert o.requires_grad and not lse.requires_grad
+    o.backward(do.cuda())
+    qr, kr, vr = (t.float().requires_grad_(True) for t in (q, k, v))
+    s = torch.einsum("bhid,bhjd->bhij", qr, kr) * scale
+    if causal:
+        s = s.masked_fill(~torch.ones(S, S, dtype=torch.bool).tril(), float("-inf"))
+    ref = torch.einsum("bhij,bhjd->bhid", torch.softmax(s, -1), vr)
+    ref.backward(do.float())
+    assert (o.detach().float().cpu() - ref.detach()).abs().max() <= 2e-2
+    for name, g, w in (("dq", qg.grad, qr.grad), ("dk", kg.grad, kr.grad), ("dv", vg.grad, vr.grad)):
+        assert g.shape == w.shape
+        _check(g, w, name)
+    # packed form
+    lens = torch.tensor([90, 40], dtype=torch.int32)
+    cu = cu_from(lens)
+    T = int(cu[-1])
+    qp, kp, vp, dop = randn((1, T, 4, D), 35), randn((1, T, 2, D), 36), randn((1, T, 2, D), 37), randn((1, T, 4, D), 38)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (qp, kp, vp))
+    ta.flash_attention(qg, kg, vg, cu.cuda()).backward(dop.cuda())
+    wq, wk, wv = orc.varlen_masked_attention_backward(qp, kp, vp, dop, cu, orc.causal_mask)
+    _check(qg.grad, wq, "packed dq")
+    _check(kg.grad, wk, "packed dk")
+    _check(vg.grad, wv, "packed dv")
+    # no gradient requested: no graph
+    with torch.no_grad():
+        assert not ta.flash_attention(qg, kg, vg, cu.cuda()).requires_grad

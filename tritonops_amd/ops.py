@@ -213,6 +213,27 @@ class flash_attn_triton(torch.autograd.Function):
         return dq, dk, dv, None
 
 
+class _FlashAttention(torch.autograd.Function):
+    """Autograd path of flash_attention(): q, k, v as [X, S, H, D] views, any
+    of the forward's options; the backward is the dense backward with the same
+    mask and scale."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, bhsd):
+        o, lse = _dense_fwd(q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, True, bhsd)
+        ctx.save_for_backward(q, k, v, o, lse, cu_seq_lens)
+        ctx.opts = (scale_log2, causal, max_seq_len)
+        ctx.mark_non_differentiable(lse)
+        return o, lse
+
+    @staticmethod
+    def backward(ctx, do, _dlse):
+        q, k, v, o, lse, cu_seq_lens = ctx.saved_tensors
+        scale_log2, causal, max_seq_len = ctx.opts
+        dq, dk, dv = _dense_bwd(q, k, v, o, lse, do, cu_seq_lens, scale_log2, causal, max_seq_len)
+        return dq, dk, dv, None, None, None, None, None
+
+
 def flash_attention(q, k, v, cu_seq_lens=None, *, causal=True, softmax_scale=None,
                     return_lse=False, max_seq_len=None):
     """The entry point the reference README advertises (README.md:30-31).
@@ -225,16 +246,27 @@ def flash_attention(q, k, v, cu_seq_lens=None, *, causal=True, softmax_scale=Non
     tutorial/4.4.causal_attention.py (causal).
     `softmax_scale` is in the natural base; default D^-0.5.
     Returns o, or (o, lse2) with return_lse (lse2 [1,T,Hq] / [B,H,S]).
+    Differentiable in q, k and v (like flash_attn_triton.apply, of which the
+    README's flash_attention is an alias): when an input requires a gradient
+    the call is recorded for autograd and backward runs the dense backward.
     """
     D = q.shape[-1]
     scale = (D ** -0.5 if softmax_scale is None else float(softmax_scale)) * LOG2E
+    needs_grad = torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)
     if cu_seq_lens is not None:
-        o, lse = _dense_fwd(q, k, v, cu_seq_lens, scale, causal, max_seq_len, return_lse)
+        if needs_grad:
+            o, lse = _FlashAttention.apply(q, k, v, cu_seq_lens, scale, causal, max_seq_len, False)
+        else:
+            o, lse = _dense_fwd(q, k, v, cu_seq_lens, scale, causal, max_seq_len, return_lse)
         return (o, lse) if return_lse else o
     if q.dim() != 4:
         raise ValueError("batched form expects [B, H, S, D] tensors")
-    o, lse = _dense_fwd(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), None, scale, causal,
-                        None, return_lse, bhsd=True)
+    if needs_grad:
+        o, lse = _FlashAttention.apply(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), None, scale, causal,
+                                       None, True)
+    else:
+        o, lse = _dense_fwd(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), None, scale, causal,
+                            None, return_lse, bhsd=True)
     o = o.transpose(1, 2)  # contiguous [B,H,S,D]
     if return_lse:
         return o, lse.transpose(1, 2)
