@@ -349,12 +349,17 @@ decode_merge_kernel(const DecodeParams p, int D) {
   if (d == 0 && p.lse) p.lse[(int64_t)b * p.hq + h] = den > 0.f ? M + fast_log2(den) : -INFINITY;
 }
 
+// CUs of the current device (cached per device; 256 if the query fails)
 int decode_cu_count() {
-  int dev = 0, n = 0;
-  if (hipGetDevice(&dev) != hipSuccess ||
-      hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-    n = 256;
-  return n;
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
 }
 
 template <typename T, int D>
