@@ -247,3 +247,27 @@ def test_packed_cache_matches_batched_and_reference_oracle_layout():
     assert torch.equal(got, ref)
     want = orc.flash_attn_decoding_torch(q, k, v, lens, faithful=False)
     assert_close(got, want, TOL)
+
+
+@pytest.mark.parametrize("split_tokens", [64, 256, None])
+def test_large_ragged_batch_is_dealt_to_the_resident_waves(split_tokens):
+    """More sequences than a wavefront has lanes (the chunk-to-sequence search
+    walks the batch 64 sequences at a time), many empty ones, and far more live
+    chunks than resident waves at the small chunk sizes."""
+    import tritonops_amd as ta
+
+    B, Hq, Hkv, D = 150, 4, 2, 64
+    g = torch.Generator().manual_seed(5)
+    lens = torch.randint(0, 700, (B,), generator=g, dtype=torch.int32)
+    lens[::7] = 0
+    lens[64] = 699
+    lens[149] = 1
+    L = int(lens.max())
+    q = randn((B, Hq, D), 41)
+    k, v = _kv(B, L, Hkv, D, torch.bfloat16, 42)
+    want = orc.flash_attn_decoding_torch(q, k, v, lens, faithful=False)
+    got, lse = ta.flash_attention_decoding(q.cuda(), k.cuda(), v.cuda(), None, seq_lens=lens.cuda(),
+                                           split_tokens=split_tokens, return_lse=True)
+    assert_close(got, want, TOL, "o")
+    assert torch.count_nonzero(got[::7]) == 0
+    assert torch.isinf(lse[::7]).all() and torch.isfinite(lse[lens.cuda() > 0]).all()
