@@ -151,7 +151,7 @@ def run_dense_bwd(steps, warmup):
                      "unit": "TFLOP/s", "kernel": "bwd_delta_kernel + bwd_kernel<bf16,128,{dq,dk,dv}> (four launches)"},
         "config": {"workload": "dense causal attention bwd bf16 B=4 H=32 S=8192 D=128: dq, dk, dv from q, k, v, o, lse, do",
                    "flop_per_step": flop,
-                   "note": "the three kernels execute 14*D FLOP per pair (S three times, dP twice); the figure "
+                   "note": "the three kernels execute 16*D FLOP per pair (S three times, dP twice); the figure "
                            "counts the 10*D of a fused backward"},
     }
 
