@@ -343,3 +343,36 @@ def test_python_wrappers_refuse_cpu_tensors():
         ta.flash_attention(q, q, q, cu)
     with pytest.raises(RuntimeError, match="GPU only"):
         ta.flash_attention_decoding(q[0], q, q, cu)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    """No fallback: with the shared library absent every entry point raises."""
+    import torch
+
+    import tritonops_amd as ta
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libmi_attn.so"))
+    with pytest.raises(ImportError):
+        _lib.load()
+    x = torch.zeros((2, 128), dtype=torch.bfloat16)
+    for call in (lambda: ta.rmsnorm_fwd(x, torch.ones(128), 1e-6),
+                 lambda: ta.cross_entropy_fused_fwd(x, x, torch.zeros(2, dtype=torch.int64)),
+                 lambda: ta.flash_attention(x.view(1, 2, 1, 128), x.view(1, 2, 1, 128), x.view(1, 2, 1, 128),
+                                            torch.tensor([0, 2], dtype=torch.int32))):
+        with pytest.raises((ImportError, RuntimeError, TypeError, ValueError)):
+            call()
+
+
+def test_product_package_never_imports_the_oracle():
+    """The oracle is test infrastructure: nothing under tritonops_amd/ (nor the
+    C sources) may import, include or mention a path into oracle/."""
+    import re
+
+    pkg = os.path.join(ROOT, "tritonops_amd")
+    pat = re.compile(r"^\s*(from|import)\s+oracle\b|oracle/|from\s+\.\.?oracle", re.M)
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".cpp", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f), encoding="utf-8", errors="ignore").read()
+                assert not pat.search(text), os.path.join(dirpath, f)
