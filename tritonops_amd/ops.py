@@ -106,6 +106,8 @@ def _dense_fwd(q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, want_lse=T
     else:
         o = torch.empty((X, S, Hq, D), device=q.device, dtype=q.dtype)
         lse = torch.empty((X, S, Hq), device=q.device, dtype=torch.float32) if want_lse else None
+    if q.numel() == 0:
+        return o, lse  # no token: nothing to launch (empty tensors have no address to pass)
     a = _lib.AttnFwdArgs()
     a.struct_size = C.sizeof(a)
     a.dtype = _dtype_tag(q)
@@ -142,6 +144,8 @@ def _dense_bwd(q, k, v, o, lse, do, cu_seq_lens, scale_log2, causal, max_seq_len
                            scale_log2, causal, max_seq_len)
         return tuple(g[..., :D].contiguous() for g in grads)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    if q.numel() == 0:
+        return dq, dk, dv
     a = _lib.AttnBwdArgs()
     a.struct_size = C.sizeof(a)
     a.dtype = _dtype_tag(q)
@@ -332,6 +336,8 @@ def flash_attn_sparse_triton(q, k, v, cu_seqlens, softmax_scale=None, local_wind
         row_ptr, col_idx, csr_strides = _masks.block_mask_to_csr(block_mask, q.device)
         if row_ptr.shape[-1] - 1 < nqb:
             raise ValueError("block mask covers %d query blocks, sequences need %d" % (row_ptr.shape[-1] - 1, nqb))
+    if q.numel() == 0:
+        return o, lse
     a = _lib.AttnSparseArgs()
     a.struct_size = C.sizeof(a)
     a.dtype = _dtype_tag(q)
@@ -372,6 +378,13 @@ def _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, re
     Hkv = k.shape[2]
     o = torch.empty((B, Hq, D), device=q.device, dtype=q.dtype)
     lse = torch.empty((B, Hq), device=q.device, dtype=torch.float32) if return_lse else None
+    if q.numel() == 0:
+        return (o, lse) if return_lse else o
+    if k.numel() == 0:  # an empty cache: every sequence has length 0
+        o.zero_()
+        if return_lse:
+            lse.fill_(float("-inf"))
+        return (o, lse) if return_lse else o
     a = _lib.DecodeArgs()
     a.struct_size = C.sizeof(a)
     a.dtype = _dtype_tag(q)
