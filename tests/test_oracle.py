@@ -22,7 +22,7 @@ def f32(shape, seed):
 
 # ---------------------------------------------------------------- dense [B,H,N,D]
 def test_config1_dense_noncausal_fp32_cpu():
-    """BASELINE config 1: B=1,H=4,S=256,D=64 fp32, scale 1/8, non-causal."""
+    """The CPU-runnable benchmark configuration: B=1, H=4, S=256, D=64 fp32, scale 1/8, non-causal."""
     q, k, v = (f32((1, 4, 256, 64), s) for s in (0, 1, 2))
     o = orc.full_attention(q, k, v)
     assert o.shape == (1, 4, 256, 64) and o.dtype == torch.float32
