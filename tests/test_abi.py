@@ -210,10 +210,11 @@ def test_split_heuristic(lib):
     f = lib.mi_decode_choose_split_tokens
     for args in [(64, 8, 32768, 256), (1, 1, 100, 256), (1, 8, 131072, 256), (512, 8, 4096, 256), (0, 0, 0, 0)]:
         t = f(*args)
-        assert t % 64 == 0 and 64 <= t <= 4096
-    assert f(64, 8, 32768, 256) <= 4096
-    assert f(1, 1, 1 << 20, 256) == 256          # one sequence: as many chunks as allowed
-    assert f(4096, 8, 4096, 256) == 4096         # plenty of sequences: one chunk each
+        assert t % 64 == 0 and 64 <= t <= 2048
+    assert f(64, 8, 32768, 256) == 2048          # plenty of work: the longest chunk
+    assert f(1, 8, 32768, 256) == 512            # little work: the shortest chunk worth a partial result
+    assert f(4, 8, 32768, 256) == 1024           # in between: about half a resident round's share
+    assert f(1, 1, 1 << 20, 256) == 1024
 
 
 def test_backward_and_rmsnorm_validation(lib):
