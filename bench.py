@@ -108,7 +108,7 @@ def run_dense_causal(steps, warmup):
         "name": "dense_causal", "ms_per_step": ms, "kernel_ms": kms,
         "metric": "attn_fwd_tflops", "unit": "TFLOP/s", "value": flop / (ms * 1e-3) / 1e12,
         "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "kernel": "prefill_kernel<bf16,128,dense>"},
+                     "unit": "TFLOP/s", "kernel": "dense_kernel<bf16,128>"},
         "config": {"workload": "dense causal flash-attention fwd bf16 B=4 H=32 S=8192 D=128, o bf16 + lse fp32",
                    "flop_per_step": flop, "flop_reference_convention_4BHS2D": 4.0 * B * H * S * S * D},
     }
@@ -260,7 +260,7 @@ def run_block_sparse(steps, warmup):
         "name": "block_sparse", "ms_per_step": ms, "kernel_ms": kms,
         "metric": "sparse_attn_fwd_tflops", "unit": "TFLOP/s", "value": flop / (ms * 1e-3) / 1e12,
         "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "kernel": "prefill_kernel<bf16,128,sparse>"},
+                     "unit": "TFLOP/s", "kernel": "sparse_kernel<bf16,128>"},
         "config": {"workload": "block-sparse causal fwd bf16 B=2 H=16 S=16384 D=128, 64x64 blocks, band 8 + 4 sink + 10%% (%d live blocks)" % live,
                    "flop_per_step": flop,
                    "kv_tile_bytes_per_step": float(live * 64 * D * 2 * 2 * B * H),

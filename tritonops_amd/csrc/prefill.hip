@@ -7,8 +7,9 @@
 // (global_load_lds_dwordx4: no staging registers, no ds_write), one barrier
 // per tile.  Block-sparse: 32-key tiles, two stages, one launch per item, each
 // wavefront runs compute_tile() on its 32 rows.  Dense: 64-key tiles, four
-// stages, a persistent grid that walks the items, and a software pipeline over
-// half tiles inside each wavefront (see the dense branch of prefill_item).
+// stages, a persistent grid that walks the items and requests the first tiles
+// of its next item before it writes out the current one, and a software
+// pipeline over half tiles inside each wavefront (see dense_kernel).
 //
 // Replaces flash_attn_fwd_kernel of flash_attn_triton/flash_attn_triton.py
 // :52-180 (dense) and flash_attn_triton/flash_attn_sparse_attn_triton.py
@@ -31,96 +32,224 @@ using ic = std::integral_constant<int, V>;
 // vmcnt(N) expcnt(7) lgkmcnt(15) for s_waitcnt on gfx9-family encodings
 constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
 
-// NW wavefronts per workgroup, NS LDS stages (tiles in flight + the one in
-// use), TN keys per tile (64, or 32 so that more workgroups fit one CU's LDS).
 extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
-// One work item: the q tile that logical workgroup id `bid` stands for.
-template <typename T, int D, int NW, int NS, int TN, bool SPARSE>
-__device__ __forceinline__ void prefill_item(const PrefillParams p, const int bid) {
+// Where one work item lives: (sequence, heads, q tile), the sequence length and
+// the element offsets of the sequence's first token in each tensor.
+struct ItemGeo {
+  int b, kvh, h, qt, len;
+  int64_t q_off, k_off, v_off, o_off, lse_off;
+};
+
+// Work item id -> geometry; false when the q tile (BM rows) starts past the end
+// of its sequence.  Consecutive ids are dealt round-robin to the 8 XCDs, each
+// with a private L2: give every XCD whole (sequence, kv-head) units so their
+// K/V stay in one L2, and walk the q tiles of a unit from the longest (last)
+// to the shortest.
+template <int BM>
+__device__ __forceinline__ bool item_geo(const PrefillParams& p, const int bid, ItemGeo& g) {
+  const int gqa = p.hq / p.hkv;
+  const int per_unit = p.n_qtiles * gqa;
+  const int n_units = p.batch * p.hkv;
+  int unit, s;
+  if ((n_units & 7) == 0) {
+    const int xcd = bid & 7, slot = bid >> 3;
+    unit = (slot / per_unit) * 8 + xcd;
+    s = slot % per_unit;
+  } else {
+    unit = bid / per_unit;
+    s = bid % per_unit;
+  }
+  g.qt = p.n_qtiles - 1 - s / gqa;
+  g.b = unit / p.hkv;
+  g.kvh = unit % p.hkv;
+  g.h = g.kvh * gqa + s % gqa;
+  if (p.cu) {
+    const int start = p.cu[g.b];
+    g.len = p.cu[g.b + 1] - start;
+    g.q_off = start * p.q_ss;
+    g.k_off = start * p.k_ss;
+    g.v_off = start * p.v_ss;
+    g.o_off = start * p.o_ss;
+    g.lse_off = start * p.lse_ss;
+  } else {
+    g.len = p.max_seqlen;
+    g.q_off = g.b * p.q_sb;
+    g.k_off = g.b * p.k_sb;
+    g.v_off = g.b * p.v_sb;
+    g.o_off = g.b * p.o_sb;
+    g.lse_off = g.b * p.lse_sb;
+  }
+  return g.qt * BM < g.len;
+}
+
+// K and V of one (sequence, kv-head): first token, as pointers and as 64-bit
+// values the compiler knows to be wave-uniform, and the sequence length.
+template <typename T>
+struct KvSrc {
+  const T *kp, *vp;
+  uint64_t k_base, v_base;
+  int len;
+};
+
+// Direct-to-LDS loads of KV tiles.  NW wavefronts share a tile of TN keys; the
+// ring has NS stages (NS K tiles, then NS V tiles).  Instruction t of a wave
+// fills the 1 KiB of LDS that holds tile rows RPI*(wave + NW*t) .. +RPI-1:
+// lane i's 16 bytes land in slot i of that KiB, i.e. row drow = i / SLOTS, slot
+// dslot = i % SLOTS, which must receive logical chunk dslot ^ swz(row) of that
+// row.
+template <typename T, int D, int NW, int NS, int TN>
+struct TileDma {
   using G = RowGeom<D>;
   using F = SwizzledFrags<D>;
-  constexpr int BM = 32 * NW;
-  constexpr int TILEB = TN * F::ROWB;   // one K or V tile
-  constexpr int VBASE = NS * TILEB;         // LDS: NS K tiles, then NS V tiles
-  constexpr int RPI = 1024 / F::ROWB;       // tile rows filled by one direct-to-LDS instruction
-  constexpr int NINST = TN / RPI;       // such instructions per tensor per tile
-  constexpr int IPW = NINST / NW;           // ... per wavefront
+  static constexpr int TILEB = TN * F::ROWB;  // one K or V tile
+  static constexpr int VBASE = NS * TILEB;    // first V tile
+  static constexpr int RPI = 1024 / F::ROWB;  // tile rows filled by one instruction
+  static constexpr int NINST = TN / RPI;      // instructions per tensor per tile
+  static constexpr int IPW = NINST / NW;      // ... per wavefront
   static_assert(NINST % NW == 0, "tile rows must split evenly over the waves");
-  constexpr int OROWB = D * 2 + 16;         // epilogue staging row
+
+  uint32_t lds0;
+  int wave, lane;
+  int64_t k_rowb, v_rowb;      // bytes between keys
+  uint32_t k_pitch, v_pitch;   // the same, wave-uniform
+  uint32_t koff[IPW], voff[IPW];
+
+  static __device__ __forceinline__ uint64_t uniform64(uint64_t x) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)x);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(x >> 32));
+    return ((uint64_t)hi << 32) | lo;
+  }
+  // The load is issued from inline assembly on purpose: the compiler then does
+  // not know that LDS writes are in flight.  When it knows, it makes every
+  // transposing LDS read wait for ALL outstanding loads (vmcnt(0)), the tile
+  // requested a moment ago included, which turns the multi-stage pipeline into
+  // a synchronous copy.  Completion is tracked by hand instead: a wave's loads
+  // retire in order, so "at most n younger loads outstanding" (counted vmcnt
+  // waits) followed by the workgroup barrier publishes a tile.  M0 carries the
+  // LDS byte address of the 1 KiB slab.
+  static __device__ __forceinline__ void dma16(const char* g, uint32_t slab_u) {
+    const uint32_t slab = (uint32_t)__builtin_amdgcn_readfirstlane(slab_u);  // uniform by construction
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(g), "s"(slab)
+                 : "memory");
+  }
+
+  __device__ __forceinline__ void init(const PrefillParams& p, int lane_, int wave_) {
+    lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem);
+    wave = wave_;
+    lane = lane_;
+    const int drow = lane / F::SLOTS, dslot = lane % F::SLOTS;
+    k_rowb = p.k_ss * 2;
+    v_rowb = p.v_ss * 2;
+    k_pitch = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)k_rowb);
+    v_pitch = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)v_rowb);
+    // A tile load address is (uniform tensor base + uniform tile offset), both
+    // kept in scalar registers, plus a per-lane 32-bit offset that is fixed for
+    // the whole launch: two vector instructions per load instead of a 64-bit
+    // multiply-add chain.
+#pragma unroll
+    for (int t = 0; t < IPW; ++t) {
+      const int r = RPI * (wave + NW * t) + drow;
+      koff[t] = (uint32_t)r * k_pitch + (uint32_t)(dslot ^ F::swz_k(r)) * 16u;
+      voff[t] = (uint32_t)r * v_pitch + (uint32_t)(dslot ^ F::swz_v(r)) * 16u;
+    }
+  }
+
+  static __device__ __forceinline__ KvSrc<T> source(const T* kp, const T* vp, int len) {
+    KvSrc<T> s;
+    s.kp = kp;
+    s.vp = vp;
+    s.k_base = uniform64((uint64_t)(uintptr_t)kp);
+    s.v_base = uniform64((uint64_t)(uintptr_t)vp);
+    s.len = len;
+    return s;
+  }
+
+  // keys k0 .. k0+TN-1 of `s` into stage ST
+  template <int ST>
+  __device__ __forceinline__ void tile(const KvSrc<T>& s, int k0) const {
+    const uint32_t sK = lds0 + ST * TILEB;
+    const uint32_t sV = lds0 + VBASE + ST * TILEB;
+    // (lane coordinates from an opaque copy: nothing derived from them is
+    // worth a register across the tile loop)
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    const int drow = ln / F::SLOTS, dslot = ln % F::SLOTS;
+    if (k0 + TN <= s.len) {
+      // whole tile inside the sequence
+      const uint32_t k0u = (uint32_t)__builtin_amdgcn_readfirstlane(k0);
+      const uint64_t kt_u = s.k_base + (uint64_t)k0u * k_pitch, vt_u = s.v_base + (uint64_t)k0u * v_pitch;
+#pragma unroll
+      for (int t = 0; t < IPW; ++t) {
+        const int inst = wave + NW * t;
+        const int r = RPI * inst + drow;
+        const int kc = dslot ^ F::swz_k(r), vc = dslot ^ F::swz_v(r);
+        if (D != 96 || kc < G::NCH) dma16(reinterpret_cast<const char*>(kt_u + koff[t]), sK + inst * 1024);
+        if (D != 96 || vc < G::NCH) dma16(reinterpret_cast<const char*>(vt_u + voff[t]), sV + inst * 1024);
+      }
+    } else {
+      // rows past the sequence end re-read its last row (masked later)
+      const char* kt = reinterpret_cast<const char*>(s.kp) + k0 * k_rowb;
+      const char* vt = reinterpret_cast<const char*>(s.vp) + k0 * v_rowb;
+#pragma unroll
+      for (int t = 0; t < IPW; ++t) {
+        const int inst = wave + NW * t;
+        const int r = RPI * inst + drow;
+        const int kc = dslot ^ F::swz_k(r), vc = dslot ^ F::swz_v(r);
+        const int64_t rr = min(k0 + r, s.len - 1) - k0;
+        if (D != 96 || kc < G::NCH) dma16(kt + rr * k_rowb + kc * 16, sK + inst * 1024);
+        if (D != 96 || vc < G::NCH) dma16(vt + rr * v_rowb + vc * 16, sV + inst * 1024);
+      }
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------
+// Block-sparse: one workgroup of NW wavefronts per q tile of 32*NW rows (one
+// block row), TN-key tiles of the listed blocks through an NS-stage ring.
+template <typename T, int D, int NW, int NS, int TN>
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2)))
+sparse_kernel(const PrefillParams p) {
+  using G = RowGeom<D>;
+  using F = SwizzledFrags<D>;
+  using DMA = TileDma<T, D, NW, NS, TN>;
+  constexpr int BM = 32 * NW;
+  constexpr int TILEB = DMA::TILEB, VBASE = DMA::VBASE, IPW = DMA::IPW;
+  constexpr int OROWB = D * 2 + 16;  // epilogue staging row
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-  // ---- workgroup -> (sequence, head, q tile).  Consecutive workgroup ids are
-  // dealt round-robin to the 8 XCDs, each with a private L2: give every XCD
-  // whole (sequence, kv-head) units so their K/V stay in one L2, and walk the
-  // q tiles of a unit from the longest (last) to the shortest.
-  const int gqa = p.hq / p.hkv;
-  const int per_unit = p.n_qtiles * gqa;
-  const int n_units = p.batch * p.hkv;
-  int unit, s;
-  {
-    if ((n_units & 7) == 0) {
-      const int xcd = bid & 7, slot = bid >> 3;
-      unit = (slot / per_unit) * 8 + xcd;
-      s = slot % per_unit;
-    } else {
-      unit = bid / per_unit;
-      s = bid % per_unit;
-    }
-  }
-  const int qt = p.n_qtiles - 1 - s / gqa;
-  const int b = unit / p.hkv;
-  const int kvh = unit % p.hkv;
-  const int h = kvh * gqa + s % gqa;
-
-  int len;
-  int64_t q_off, k_off, v_off, o_off, lse_off;
-  if (p.cu) {
-    const int start = p.cu[b];
-    len = p.cu[b + 1] - start;
-    q_off = start * p.q_ss;
-    k_off = start * p.k_ss;
-    v_off = start * p.v_ss;
-    o_off = start * p.o_ss;
-    lse_off = start * p.lse_ss;
-  } else {
-    len = p.max_seqlen;
-    q_off = b * p.q_sb;
-    k_off = b * p.k_sb;
-    v_off = b * p.v_sb;
-    o_off = b * p.o_sb;
-    lse_off = b * p.lse_sb;
-  }
+  ItemGeo g;
+  if (!item_geo<BM>(p, blockIdx.x, g)) return;
+  const int len = g.len, qt = g.qt, h = g.h;
   const int q0 = qt * BM;
-  if (q0 >= len) return;
-
-  const T* qp = reinterpret_cast<const T*>(p.q) + q_off + h * p.q_sh;
-  const T* kp = reinterpret_cast<const T*>(p.k) + k_off + kvh * p.k_sh;
-  const T* vp = reinterpret_cast<const T*>(p.v) + v_off + kvh * p.v_sh;
-  T* op = reinterpret_cast<T*>(p.o) + o_off + h * p.o_sh;
+  const T* qp = reinterpret_cast<const T*>(p.q) + g.q_off + h * p.q_sh;
+  T* op = reinterpret_cast<T*>(p.o) + g.o_off + h * p.o_sh;
 
   F fr;
   fr.init(lane, (uint32_t)(uintptr_t)smem, VBASE);
+  DMA dma;
+  dma.init(p, lane, wave);
+  const KvSrc<T> kv = DMA::source(reinterpret_cast<const T*>(p.k) + g.k_off + g.kvh * p.k_sh,
+                                  reinterpret_cast<const T*>(p.v) + g.v_off + g.kvh * p.v_sh, len);
   const int q0w = q0 + 32 * wave;
   const int qrow = q0w + fr.lq;
 
-  // ---- tile list
-  int n_tiles;
-  const int32_t* cols = nullptr;
-  if constexpr (SPARSE) {
-    const int32_t* rp = p.row_ptr + b * p.rp_sb + h * p.rp_sh;
-    // (values loaded through vector memory: tell the compiler they are uniform)
-    const int beg = __builtin_amdgcn_readfirstlane(rp[qt]);
-    n_tiles = __builtin_amdgcn_readfirstlane(rp[qt + 1] - beg) * (kTileN / TN);  // a 64-key block is TN-key tiles
-    cols = p.col_idx + b * p.ci_sb + h * p.ci_sh + beg;
-  } else {
-    static_assert(SPARSE || TN == kTileN, "dense kernel walks 64-key tiles");
-    n_tiles = (len + TN - 1) / TN;
-    if (p.causal) n_tiles = min(n_tiles, (q0 + BM + TN - 1) / TN);
-  }
+  // ---- tile list: a listed 64-key block is walked as kTileN / TN tiles
+  const int32_t* rp = p.row_ptr + g.b * p.rp_sb + h * p.rp_sh;
+  // (values loaded through vector memory: tell the compiler they are uniform)
+  const int beg = __builtin_amdgcn_readfirstlane(rp[qt]);
+  const int n_tiles = __builtin_amdgcn_readfirstlane(rp[qt + 1] - beg) * (kTileN / TN);
+  const int32_t* cols = p.col_idx + g.b * p.ci_sb + h * p.ci_sh + beg;
+  // first key of tile `it`
+  auto tile_k0 = [&](int it) __attribute__((always_inline)) -> int {
+    constexpr int PER = kTileN / TN;
+    return __builtin_amdgcn_readfirstlane(cols[it / PER]) * kTileN + (it % PER) * TN;
+  };
 
   // ---- Q^T operands: lane (query lq, half lh) holds d = 16c + 8lh .. +7
   i32x4 Qf[G::KSTEPS];
@@ -135,253 +264,424 @@ __device__ __forceinline__ void prefill_item(const PrefillParams p, const int bi
   for (int db = 0; db < G::NDB; ++db) O[db] = (f32x16){0};
   float m = -INFINITY, l = 0.f;
 
-  // ---- direct-to-LDS tile loads.  Instruction t of this wave fills the 1 KiB
-  // of LDS that holds tile rows RPI*(wave + NW*t) .. +RPI-1: lane i's 16 bytes
-  // land in slot i of that KiB, i.e. row drow = i / SLOTS, slot dslot = i %
-  // SLOTS, which must receive logical chunk dslot ^ swz(row) of that row.
-  const int drow = lane / F::SLOTS, dslot = lane % F::SLOTS;
-  const int64_t k_rowb = p.k_ss * 2, v_rowb = p.v_ss * 2;  // bytes between keys
-  // first key of tile `it` of this workgroup's list
-  auto tile_k0 = [&](int it) __attribute__((always_inline)) -> int {
-    if (!SPARSE) return it * TN;
-    constexpr int PER = kTileN / TN;
-    return __builtin_amdgcn_readfirstlane(cols[it / PER]) * kTileN + (it % PER) * TN;
-  };
-  // The load is issued from inline assembly on purpose: the compiler then does
-  // not know that LDS writes are in flight.  When it knows, it makes every
-  // transposing LDS read wait for ALL outstanding loads (vmcnt(0)), the tile
-  // requested a moment ago included, which turns the multi-stage pipeline into
-  // a synchronous copy.  Completion is tracked by hand instead: this wave's
-  // loads retire in order, so "at most n younger loads outstanding" (the
-  // counted vmcnt waits below) followed by the workgroup barrier publishes a
-  // tile.  M0 carries the LDS byte address of the 1 KiB slab.
-  const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem);
-  auto dma16 = [&](const char* g, uint32_t slab_u) __attribute__((always_inline)) {
-    const uint32_t slab = (uint32_t)__builtin_amdgcn_readfirstlane(slab_u);  // uniform by construction
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                 :
-                 : "v"(g), "s"(slab)
-                 : "memory");
-  };
-  // A tile load address is (uniform tensor base + uniform tile offset), both
-  // kept in scalar registers, plus a per-lane 32-bit offset that is fixed for
-  // the whole item: two vector instructions per load instead of a 64-bit
-  // multiply-add chain.
-  auto uniform64 = [](uint64_t x) __attribute__((always_inline)) -> uint64_t {
-    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)x);
-    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(x >> 32));
-    return ((uint64_t)hi << 32) | lo;
-  };
-  const uint32_t k_pitch = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)k_rowb);
-  const uint32_t v_pitch = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)v_rowb);
-  const uint64_t k_base = uniform64((uint64_t)(uintptr_t)kp);
-  const uint64_t v_base = uniform64((uint64_t)(uintptr_t)vp);
-  uint32_t koff[IPW], voff[IPW];
-#pragma unroll
-  for (int t = 0; t < IPW; ++t) {
-    const int r = RPI * (wave + NW * t) + drow;
-    koff[t] = (uint32_t)r * k_pitch + (uint32_t)(dslot ^ F::swz_k(r)) * 16u;
-    voff[t] = (uint32_t)r * v_pitch + (uint32_t)(dslot ^ F::swz_v(r)) * 16u;
-  }
-  auto dma_tile = [&](int k0, auto stage_c) __attribute__((always_inline)) {
+  auto step = [&](auto stage_c, int it) {
     constexpr int ST = decltype(stage_c)::value;
-    const char* kt = reinterpret_cast<const char*>(kp) + k0 * k_rowb;
-    const char* vt = reinterpret_cast<const char*>(vp) + k0 * v_rowb;
-    const uint32_t sK = lds0 + ST * TILEB;
-    const uint32_t sV = lds0 + VBASE + ST * TILEB;
-    if (k0 + TN <= len) {
-      // whole tile inside the sequence
-      const uint32_t k0u = (uint32_t)__builtin_amdgcn_readfirstlane(k0);
-      const uint64_t kt_u = k_base + (uint64_t)k0u * k_pitch, vt_u = v_base + (uint64_t)k0u * v_pitch;
+    // refill the stage that was read in the previous iteration
+    const bool refill = it + NS - 1 < n_tiles;
+    if (refill) dma.template tile<(ST + NS - 1) % NS>(kv, tile_k0(it + NS - 1));
+
+    const int k0 = tile_k0(it);
+    // whole tile above the diagonal for this wave: nothing to add
+    const bool skip = p.causal && k0 > q0w + 31;
+    if (!skip) {
+      bool need_mask = (k0 + TN > len) || (p.causal && k0 + TN - 1 > q0w);
+      const int wl = p.win_local, wg = p.win_global;
+      if (wl >= 0) need_mask = need_mask || !((k0 + TN - 1 < wg) || (q0w + 31 - k0 < wl));
+      const int causal = p.causal;
+      auto allowed = [&](int key_in_tile) -> bool {
+        const int key = k0 + key_in_tile;
+        bool ok = key < len && (!causal || key <= qrow);
+        if (wl >= 0) ok = ok && ((qrow - key < wl) || (key < wg));
+        return ok;
+      };
+      // V addresses carry VBASE inside the lane offsets (see fr.init)
+      compute_tile<T, D, TN / 32>((uint32_t)(ST * TILEB), (uint32_t)(ST * TILEB), fr, Qf, O, m, l, p.scale, need_mask, allowed);
+    }
+    // The next tile must have landed and everyone must be done with this one.
+    // This wave's loads complete in order, so it is enough that at most the
+    // loads of the NS-2 younger tiles are still in flight (2*IPW each).
+    if (refill)
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * 2 * IPW));
+    else
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    __syncthreads();
+  };
+
 #pragma unroll
-      for (int t = 0; t < IPW; ++t) {
-        const int inst = wave + NW * t;
-        const int r = RPI * inst + drow;
-        const int kc = dslot ^ F::swz_k(r), vc = dslot ^ F::swz_v(r);
-        if (D != 96 || kc < G::NCH) dma16(reinterpret_cast<const char*>(kt_u + koff[t]), sK + inst * 1024);
-        if (D != 96 || vc < G::NCH) dma16(reinterpret_cast<const char*>(vt_u + voff[t]), sV + inst * 1024);
-      }
-    } else {
-      // rows past the sequence end re-read its last row (masked later)
+  for (int s0 = 0; s0 < NS - 1; ++s0)
+    if (s0 < n_tiles) {
+      if (s0 == 0) dma.template tile<0>(kv, tile_k0(0));
+      if (s0 == 1) dma.template tile<1 % NS>(kv, tile_k0(1));
+      if (s0 == 2) dma.template tile<2 % NS>(kv, tile_k0(2));
+    }
+  // tile 0 (and the Q loads issued before it) must be complete
+  if (n_tiles >= NS - 1)
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * 2 * IPW));
+  else
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+  __syncthreads();
+
+  int it = 0;
+  for (; it + NS <= n_tiles; it += NS) {
+    step(ic<0>{}, it);
+    step(ic<1 % NS>{}, it + 1);
+    if (NS > 2) step(ic<2 % NS>{}, it + 2);
+    if (NS > 3) step(ic<3 % NS>{}, it + 3);
+  }
+  if (it < n_tiles) step(ic<0>{}, it++);
+  if (it < n_tiles) step(ic<1 % NS>{}, it++);
+  if (NS > 3 && it < n_tiles) step(ic<2 % NS>{}, it++);
+
+  // ---- epilogue: normalise, transpose through LDS, coalesced 16-byte stores
+  const float l_tot = sum_with_other_half(l);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  if (p.lse && fr.lh == 0 && qrow < len) {
+    float* lp = p.lse + g.lse_off + h * p.lse_sh;
+    lp[(int64_t)qrow * p.lse_ss] = l_tot > 0.f ? m + fast_log2(l_tot) : -INFINITY;
+  }
+  unsigned char* stage = smem + wave * 32 * OROWB;
 #pragma unroll
-      for (int t = 0; t < IPW; ++t) {
-        const int inst = wave + NW * t;
-        const int r = RPI * inst + drow;
-        const int kc = dslot ^ F::swz_k(r), vc = dslot ^ F::swz_v(r);
-        const int64_t rr = min(k0 + r, len - 1) - k0;
-        if (D != 96 || kc < G::NCH)
-          dma16(kt + rr * k_rowb + kc * 16, sK + inst * 1024);
-        if (D != 96 || vc < G::NCH)
-          dma16(vt + rr * v_rowb + vc * 16, sV + inst * 1024);
+  for (int db = 0; db < G::NDB; ++db)
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {
+      const int d = 32 * db + 8 * gq + 4 * fr.lh;
+      i32x2 w;
+      w[0] = (int)Elem<T>::pack2(O[db][4 * gq] * inv, O[db][4 * gq + 1] * inv);
+      w[1] = (int)Elem<T>::pack2(O[db][4 * gq + 2] * inv, O[db][4 * gq + 3] * inv);
+      *reinterpret_cast<i32x2*>(stage + fr.lq * OROWB + d * 2) = w;
+    }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < (32 * G::NCH + 63) / 64; ++i) {
+    const int idx = lane + 64 * i;
+    const int row = idx / G::NCH, ch = idx % G::NCH;
+    if (((32 * G::NCH) % 64 == 0 || idx < 32 * G::NCH) && q0w + row < len) {
+      const i32x4 val = *reinterpret_cast<const i32x4*>(stage + row * OROWB + ch * 16);
+      *reinterpret_cast<i32x4*>(op + (int64_t)(q0w + row) * p.o_ss + ch * 8) = val;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Dense: persistent workgroups of 8 wavefronts (256 query rows per item).
+//
+// The grid holds at most as many workgroups as the device runs at once, and
+// each walks the work item ids id, id + grid, ...: a fresh workgroup launch
+// left the CU idle for several microseconds (measured ~12 us between the end
+// of one 512-thread, 128 KiB-LDS workgroup and the first instruction of the
+// next).  Odd rounds are walked back to front within each XCD (id & 7 is
+// kept): ids run from the longest q tile of a unit to the shortest, so the
+// workgroup that drew a long tile in one round draws a short one in the next,
+// which balances causal work without a shared counter.
+//
+// Item boundary: once every wave is done with the tiles of an item, the
+// workgroup requests Q and the first NS-1 tiles of its NEXT item (stages
+// 0..NS-2) and only then normalises and writes out the current one, staging
+// the output through the last stage, so the load latency of the next item is
+// covered by the epilogue of this one; one barrier separates the two items.
+//
+// Inner loop: a software pipeline over HALF tiles (32 keys) inside each wave.
+// MFMA and softmax arithmetic overlap best when one wave's instruction stream
+// interleaves them, so at position h the wave runs two straight-line blocks:
+// the 8 MFMAs of S[h+1] = K Q^T together with half of the exp2 / sum / convert
+// work of S[h], then the 8 MFMAs of O += V^T P[h]^T together with the first
+// half of that work for S[h+1].  K of half h+1 must be in LDS while half h is
+// being finished: tile t+1 has to be visible before position 2t+1, which the
+// barrier at the top of tile t guarantees.
+template <typename T, int D>
+__global__ void __launch_bounds__(kDenseRows * 2) __attribute__((amdgpu_waves_per_eu(2)))
+dense_kernel(const PrefillParams p) {
+  constexpr int NW = kDenseRows / 32, NS = kDenseStages, TN = kTileN;
+  static_assert(NW == 8 && NS == 4 && TN == 64, "stage use at the item boundary assumes this shape");
+  using G = RowGeom<D>;
+  using F = SwizzledFrags<D>;
+  using DMA = TileDma<T, D, NW, NS, TN>;
+  constexpr int BM = 32 * NW;
+  constexpr int TILEB = DMA::TILEB, VBASE = DMA::VBASE, IPW = DMA::IPW;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  F fr;
+  fr.init(lane, (uint32_t)(uintptr_t)smem, VBASE);
+  DMA dma;
+  dma.init(p, lane, wave);
+  const int causal = p.causal;
+  const float scale = p.scale;
+
+  // ---- the items of this workgroup
+  struct Item {
+    int len, q0, n_tiles;
+    const T* qp;
+    T* op;
+    float* lp;  // LSE row of this head, or null
+    KvSrc<T> kv;
+  };
+  const int grid = gridDim.x;
+  int round = 0, base = 0;
+  // advance to the next item of this workgroup that has rows; false when there is none
+  auto next_item = [&](Item& it) __attribute__((always_inline)) -> bool {
+    while (base < p.n_items) {
+      int w = blockIdx.x;
+      if ((round & 1) && (grid & 7) == 0) w = (((grid >> 3) - 1 - (w >> 3)) << 3) | (w & 7);
+      const int bid = base + w;
+      base += grid;
+      ++round;
+      ItemGeo g;
+      if (bid < p.n_items && item_geo<BM>(p, bid, g)) {
+        it.len = g.len;
+        it.q0 = g.qt * BM;
+        it.n_tiles = (g.len + TN - 1) / TN;
+        if (causal) it.n_tiles = min(it.n_tiles, (it.q0 + BM + TN - 1) / TN);
+        it.qp = reinterpret_cast<const T*>(p.q) + g.q_off + g.h * p.q_sh;
+        it.op = reinterpret_cast<T*>(p.o) + g.o_off + g.h * p.o_sh;
+        it.lp = p.lse ? p.lse + g.lse_off + g.h * p.lse_sh : nullptr;
+        it.kv = DMA::source(reinterpret_cast<const T*>(p.k) + g.k_off + g.kvh * p.k_sh,
+                            reinterpret_cast<const T*>(p.v) + g.v_off + g.kvh * p.v_sh, g.len);
+        return true;
       }
+    }
+    return false;
+  };
+  // Q^T operands of an item (lane (query lq, half lh) holds d = 16c + 8lh .. +7)
+  // and its first NS-1 tiles; nothing waits here
+  auto request_item = [&](const Item& it, i32x4 (&Q)[G::KSTEPS]) __attribute__((always_inline)) {
+    const int row = min(it.q0 + 32 * wave + fr.lq, it.len - 1);
+    const T* qr = it.qp + (int64_t)row * p.q_ss + 8 * fr.lh;
+    // Issued from inline assembly like the tile loads, and for the same reason:
+    // a load the compiler knows about is guarded by a counted wait at its first
+    // use, and that wait would also cover the output stores issued after it.
+    // The registers are complete after the wait at the top of the item.
+#pragma unroll
+    for (int c = 0; c < G::KSTEPS; ++c)
+      asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(Q[c]) : "v"(qr), "n"(32 * c));
+    if (0 < it.n_tiles) dma.template tile<0>(it.kv, 0);
+    if (1 < it.n_tiles) dma.template tile<1>(it.kv, TN);
+    if (2 < it.n_tiles) dma.template tile<2>(it.kv, 2 * TN);
+  };
+
+  // ---- state of the item being computed
+  Item cur;
+  i32x4 Qf[G::KSTEPS];
+  f32x16 O[G::NDB];
+  float m, l;
+  int len, n_tiles, q0w, qrow, row_lim, H_w;
+  f32x16 S[2];
+  constexpr int KR = G::KSTEPS < 4 ? G::KSTEPS : 4;  // K fragments kept in flight
+  i32x4 kf[KR];  // fragments 0..KR-1 of the half that is scored next, read one block ahead
+
+  // keys of half hh that this lane's query must not see -> -inf (rare)
+  auto mask_half = [&](int hh, f32x16& Sx) __attribute__((always_inline)) {
+    const int k0h = hh * 32;
+    if ((k0h + 32 > len) || (causal && k0h + 31 > q0w)) {
+      const int t = row_lim - k0h - 8 * fr.lh;
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (16 * (r >> 3) + (r & 7) > t) Sx[r] = -INFINITY;
     }
   };
 
-  if constexpr (!SPARSE) {
-    // ---- dense: software pipeline over HALF tiles (32 keys) inside each wave.
-    // MFMA and softmax arithmetic overlap best when one wave's instruction
-    // stream interleaves them, so at position h the wave runs two straight-line
-    // blocks: the 8 MFMAs of S[h+1] = K Q^T together with half of the exp2 /
-    // sum / convert work of S[h], then the 8 MFMAs of O += V^T P[h]^T together
-    // with the first half of that work for S[h+1].  K of half h+1 must be in LDS
-    // while half h is being finished: tile t+1 has to be visible before
-    // position 2t+1, which the barrier at the top of tile t guarantees.
-    static_assert(TN == kTileN && NS >= 3, "pipelined dense path: 64-key tiles, >= 3 stages");
-    int H_w = (len + 31) / 32;                        // halves this wave works on
-    if (p.causal) H_w = min(H_w, q0w / 32 + 1);       // nothing above its own diagonal block
-    H_w = min(H_w, 2 * n_tiles);
-    if (q0w >= len) H_w = 0;                          // all rows past the sequence end
-    f32x16 S[2];
-    const int causal = p.causal;
-    const float scale = p.scale;
-    const int row_lim = causal ? min(qrow, len - 1) : len - 1;  // largest key this lane may see
-    constexpr int KR = G::KSTEPS < 4 ? G::KSTEPS : 4;  // K fragments kept in flight
-    i32x4 kf[KR];  // fragments 0..KR-1 of the half that is scored next, read one block ahead
+  // Probabilities of a half are taken against the reference point m the row
+  // already has; m is only moved (exactly, to the true running maximum) when
+  // a lane's partial row sum of a half passes kRowSumLimit or is not finite.
+  // Any reference point gives the same o and lse, so the common path needs
+  // no row maximum at all: 7 vector instructions per pair of scores.
+  constexpr float kRowSumLimit = 4096.f;  // probabilities stay below 2^12: far inside bf16 / fp32 range
+  uint32_t Pb[2][8];  // packed probabilities of the half in S[0] / S[1]
+  float rsv[2];       // their partial row sums (this lane's 16 keys)
+  float e_p0, e_u1;   // first element done, second element scaled: carried between two slices
+  auto exp_first = [&](const f32x16& Sx, int i, float m_neg) __attribute__((always_inline)) {
+    e_p0 = fast_exp2(fmaf(Sx[2 * i], scale, m_neg));
+    e_u1 = fmaf(Sx[2 * i + 1], scale, m_neg);
+  };
+  auto exp_second = [&](int i, uint32_t (&Pd)[8], float& rs) __attribute__((always_inline)) {
+    const float p1 = fast_exp2(e_u1);
+    rs += e_p0 + p1;
+    Pd[i] = Elem<T>::pack2(e_p0, p1);
+  };
+  // rare: bring m to the exact running maximum including the half in Sx,
+  // rescale l and O, and redo the probabilities of that half
+  auto exact_fix = [&](const f32x16& Sx, uint32_t (&Pd)[8], float& rs) __attribute__((always_inline)) {
+    float mx = Sx[0];
+#pragma unroll
+    for (int r = 1; r < 16; ++r) mx = fmaxf(mx, Sx[r]);
+    mx = max_with_other_half(mx);
+    const float m_new = fmaxf(m, mx * scale);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // no key seen yet: l and O are 0
+    const float alpha = fast_exp2(m - m_safe);
+    l *= alpha;
+#pragma unroll
+    for (int db = 0; db < G::NDB; ++db) O[db] *= alpha;
+    m = m_new;
+    rs = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float p0 = fast_exp2(fmaf(Sx[2 * i], scale, -m_safe));
+      const float p1 = fast_exp2(fmaf(Sx[2 * i + 1], scale, -m_safe));
+      rs += p0 + p1;
+      Pd[i] = Elem<T>::pack2(p0, p1);
+    }
+  };
 
-    // keys of half hh that this lane's query must not see -> -inf (rare)
-    auto mask_half = [&](int hh, f32x16& Sx) __attribute__((always_inline)) {
-      const int k0h = hh * 32;
-      if ((k0h + 32 > len) || (causal && k0h + 31 > q0w)) {
-        const int t = row_lim - k0h - 8 * fr.lh;
+  // Position h.  Entry state: S[h&1] holds the scores of half h and the
+  // probabilities of its first 8 keys per lane are done; kf holds the first
+  // K fragments of half h+1.
+  //   block A: [MFMAs of S(h+1) = K Q^T]      with [exp2 / sum / pack of the last 8 keys of S(h)]
+  //   check  : row sums sane? else exact_fix (rare)
+  //   block B: [MFMAs of O += V^T P(h)^T]    with [exp2 / sum / pack of the first 8 keys of S(h+1)]
+  // so every MFMA has three or four vector instructions behind it.
+  // sched_barrier(0) after each slice pins the interleaving: one MFMA, the
+  // LDS reads for a slice four positions ahead, and those vector instructions.
+  auto half_step = [&](auto j_c, int h) __attribute__((always_inline)) {
+    constexpr int J = decltype(j_c)::value;  // h % (2 NS)
+    if (h >= H_w) return;
+    constexpr int TS = J / 2, KB = J & 1;    // stage of tile h/2, which half of it
+    constexpr int KS = KB == 0 ? TS : (TS + 1) % NS;      // stage holding K of half h+1
+    constexpr uint32_t KOFF = KS * TILEB, VOFF = TS * TILEB;
+    constexpr uint32_t K2OFF = ((TS + 1) % NS) * TILEB;   // stage holding K of half h+2
+    f32x16& Sc = S[KB];
+    f32x16& Sn = S[KB ^ 1];
+    uint32_t (&Pc)[8] = Pb[KB];
+    uint32_t (&Pn)[8] = Pb[KB ^ 1];
+    const float m_neg = (m == -INFINITY) ? 0.f : -m;
+    i32x4 vf[G::NDB];
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          if (16 * (r >> 3) + (r & 7) > t) Sx[r] = -INFINITY;
+    for (int c = 0; c < 8; ++c) {
+      if (c < G::KSTEPS) {
+        const f32x16 acc = (c == 0) ? (f32x16){0} : Sn;
+        Sn = Elem<T>::mfma(kf[c % KR], Qf[c], acc);
+        if (c + KR < G::KSTEPS) kf[c % KR] = fr.load_k(KOFF, KB ^ 1, c + KR);
       }
-    };
+      if (c >= 8 - G::NDB) vf[c - (8 - G::NDB)] = fr.load_v(VOFF, 2 * KB, c - (8 - G::NDB));
+      if ((c & 1) == 0)
+        exp_first(Sc, 4 + c / 2, m_neg);
+      else
+        exp_second(4 + c / 2, Pc, rsv[KB]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // keep the exponentials in this block (they would otherwise sink below
+    // the branches that follow, away from the MFMAs they are meant to overlap)
+    asm volatile("" : "+v"(Pc[4]), "+v"(Pc[5]), "+v"(Pc[6]), "+v"(Pc[7]), "+v"(rsv[KB]));
+    if (__builtin_amdgcn_ballot_w64(!(rsv[KB] <= kRowSumLimit)) != 0) exact_fix(Sc, Pc, rsv[KB]);
+    l += rsv[KB];
+    mask_half(h + 1, Sn);
+    const float m_neg2 = (m == -INFINITY) ? 0.f : -m;
+    rsv[KB ^ 1] = 0.f;
+#pragma unroll
+    for (int sl = 0; sl < 8; ++sl) {
+      if (sl < 2 * G::NDB) {
+        const int kk = sl / G::NDB, db = sl % G::NDB;
+        const i32x4 pf = {(int)Pc[4 * kk], (int)Pc[4 * kk + 1], (int)Pc[4 * kk + 2], (int)Pc[4 * kk + 3]};
+        O[db] = Elem<T>::mfma(vf[db], pf, O[db]);
+        if (kk == 0) vf[db] = fr.load_v(VOFF, 2 * KB + 1, db);
+      }
+      if (sl >= 4 && sl - 4 < KR) kf[sl - 4] = fr.load_k(K2OFF, KB, sl - 4);
+      // (for the last half of a wave Sn holds scores of stale LDS contents: the results are never used)
+      if ((sl & 1) == 0)
+        exp_first(Sn, sl / 2, m_neg2);
+      else
+        exp_second(sl / 2, Pn, rsv[KB ^ 1]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("" : "+v"(Pn[0]), "+v"(Pn[1]), "+v"(Pn[2]), "+v"(Pn[3]), "+v"(rsv[KB ^ 1]));
+  };
 
-    // Probabilities of a half are taken against the reference point m the row
-    // already has; m is only moved (exactly, to the true running maximum) when
-    // a lane's partial row sum of a half passes kRowSumLimit or is not finite.
-    // Any reference point gives the same o and lse, so the common path needs
-    // no row maximum at all: 7 vector instructions per pair of scores.
-    constexpr float kRowSumLimit = 4096.f;  // probabilities stay below 2^12: far inside bf16 / fp32 range
-    uint32_t Pb[2][8];  // packed probabilities of the half in S[0] / S[1]
-    float rsv[2];       // their partial row sums (this lane's 16 keys)
-    float e_p0, e_u1;   // first element done, second element scaled: carried between two slices
-    auto exp_first = [&](const f32x16& Sx, int i, float m_neg) __attribute__((always_inline)) {
-      e_p0 = fast_exp2(fmaf(Sx[2 * i], scale, m_neg));
-      e_u1 = fmaf(Sx[2 * i + 1], scale, m_neg);
-    };
-    auto exp_second = [&](int i, uint32_t (&Pd)[8], float& rs) __attribute__((always_inline)) {
-      const float p1 = fast_exp2(e_u1);
-      rs += e_p0 + p1;
-      Pd[i] = Elem<T>::pack2(e_p0, p1);
-    };
-    // rare: bring m to the exact running maximum including the half in Sx,
-    // rescale l and O, and redo the probabilities of that half
-    auto exact_fix = [&](const f32x16& Sx, uint32_t (&Pd)[8], float& rs) __attribute__((always_inline)) {
-      float mx = Sx[0];
-#pragma unroll
-      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, Sx[r]);
-      mx = max_with_other_half(mx);
-      const float m_new = fmaxf(m, mx * scale);
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;  // no key seen yet: l and O are 0
-      const float alpha = fast_exp2(m - m_safe);
-      l *= alpha;
-#pragma unroll
-      for (int db = 0; db < G::NDB; ++db) O[db] *= alpha;
-      m = m_new;
-      rs = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float p0 = fast_exp2(fmaf(Sx[2 * i], scale, -m_safe));
-        const float p1 = fast_exp2(fmaf(Sx[2 * i + 1], scale, -m_safe));
-        rs += p0 + p1;
-        Pd[i] = Elem<T>::pack2(p0, p1);
-      }
-    };
-
-    // Position h.  Entry state: S[h&1] holds the scores of half h and the
-    // probabilities of its first 8 keys per lane are done; kf holds the first
-    // K fragments of half h+1.
-    //   block A: [MFMAs of S(h+1) = K Q^T]      with [exp2 / sum / pack of the last 8 keys of S(h)]
-    //   check  : row sums sane? else exact_fix (rare)
-    //   block B: [MFMAs of O += V^T P(h)^T]    with [exp2 / sum / pack of the first 8 keys of S(h+1)]
-    // so every MFMA has three or four vector instructions behind it.
-    // sched_barrier(0) after each slice pins the interleaving: one MFMA, the
-    // LDS reads for a slice four positions ahead, and those vector instructions.
-    auto half_step = [&](auto j_c, int h) __attribute__((always_inline)) {
-      constexpr int J = decltype(j_c)::value;  // h % (2 NS)
-      if (h >= H_w) return;
-      constexpr int TS = J / 2, KB = J & 1;    // stage of tile h/2, which half of it
-      constexpr int KS = KB == 0 ? TS : (TS + 1) % NS;      // stage holding K of half h+1
-      constexpr uint32_t KOFF = KS * TILEB, VOFF = TS * TILEB;
-      constexpr uint32_t K2OFF = ((TS + 1) % NS) * TILEB;   // stage holding K of half h+2
-      f32x16& Sc = S[KB];
-      f32x16& Sn = S[KB ^ 1];
-      uint32_t (&Pc)[8] = Pb[KB];
-      uint32_t (&Pn)[8] = Pb[KB ^ 1];
-      const float m_neg = (m == -INFINITY) ? 0.f : -m;
-      i32x4 vf[G::NDB];
-#pragma unroll
-      for (int c = 0; c < 8; ++c) {
-        if (c < G::KSTEPS) {
-          const f32x16 acc = (c == 0) ? (f32x16){0} : Sn;
-          Sn = Elem<T>::mfma(kf[c % KR], Qf[c], acc);
-          if (c + KR < G::KSTEPS) kf[c % KR] = fr.load_k(KOFF, KB ^ 1, c + KR);
-        }
-        if (c >= 8 - G::NDB) vf[c - (8 - G::NDB)] = fr.load_v(VOFF, 2 * KB, c - (8 - G::NDB));
-        if ((c & 1) == 0)
-          exp_first(Sc, 4 + c / 2, m_neg);
-        else
-          exp_second(4 + c / 2, Pc, rsv[KB]);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      // keep the exponentials in this block (they would otherwise sink below
-      // the branches that follow, away from the MFMAs they are meant to overlap)
-      asm volatile("" : "+v"(Pc[4]), "+v"(Pc[5]), "+v"(Pc[6]), "+v"(Pc[7]), "+v"(rsv[KB]));
-      if (__builtin_amdgcn_ballot_w64(!(rsv[KB] <= kRowSumLimit)) != 0) exact_fix(Sc, Pc, rsv[KB]);
-      l += rsv[KB];
-      mask_half(h + 1, Sn);
-      const float m_neg2 = (m == -INFINITY) ? 0.f : -m;
-      rsv[KB ^ 1] = 0.f;
-#pragma unroll
-      for (int sl = 0; sl < 8; ++sl) {
-        if (sl < 2 * G::NDB) {
-          const int kk = sl / G::NDB, db = sl % G::NDB;
-          const i32x4 pf = {(int)Pc[4 * kk], (int)Pc[4 * kk + 1], (int)Pc[4 * kk + 2], (int)Pc[4 * kk + 3]};
-          O[db] = Elem<T>::mfma(vf[db], pf, O[db]);
-          if (kk == 0) vf[db] = fr.load_v(VOFF, 2 * KB + 1, db);
-        }
-        if (sl >= 4 && sl - 4 < KR) kf[sl - 4] = fr.load_k(K2OFF, KB, sl - 4);
-        // (for the last half of a wave Sn holds scores of stale LDS contents: the results are never used)
-        if ((sl & 1) == 0)
-          exp_first(Sn, sl / 2, m_neg2);
-        else
-          exp_second(sl / 2, Pn, rsv[KB ^ 1]);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      asm volatile("" : "+v"(Pn[0]), "+v"(Pn[1]), "+v"(Pn[2]), "+v"(Pn[3]), "+v"(rsv[KB ^ 1]));
-    };
-
-    // tile t: barrier (tile t+1 visible, stage of tile t-1 free), refill, two halves
-    auto tile_iter = [&](auto ts_c, int t) __attribute__((always_inline)) {
-      constexpr int TS = decltype(ts_c)::value;
+  // tile t: barrier (tile t+1 visible, stage of tile t-1 free), refill, two halves.
+  // (Tile 0: the item's first barrier has done all of that.)
+  auto tile_iter = [&](auto ts_c, int t) __attribute__((always_inline)) {
+    constexpr int TS = decltype(ts_c)::value;
+    if (t > 0) {
       // tile t+1 was requested NS-2 iterations ago; at most NS-3 younger tiles may still fly
       if (t + NS - 2 < n_tiles)
         __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 3) * 2 * IPW));
       else
         __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
       __syncthreads();
-      if (t + NS - 1 < n_tiles) dma_tile(tile_k0(t + NS - 1), ic<(TS + NS - 1) % NS>{});
-      half_step(ic<2 * TS>{}, 2 * t);
-      half_step(ic<2 * TS + 1>{}, 2 * t + 1);
-    };
+      if (t + NS - 1 < n_tiles) dma.template tile<(TS + NS - 1) % NS>(cur.kv, (t + NS - 1) * TN);
+    }
+    half_step(ic<2 * TS>{}, 2 * t);
+    half_step(ic<2 * TS + 1>{}, 2 * t + 1);
+  };
 
+  // ---- normalise, transpose through LDS, coalesced 16-byte stores; LSE from
+  // half the lanes.  The staging area is the LAST stage (first four waves in
+  // its K tile, the others in its V tile) because the other stages are being
+  // filled for the next item; a wave stages and stores its 32 rows in two
+  // passes of up to 64 columns.  Only the wave itself reads what it staged and
+  // a wave's LDS accesses execute in order, so no barrier is needed.
+  constexpr int DBP = (G::NDB + 1) / 2;  // 32-column blocks of O per pass
+  constexpr int SROW = DBP * 64;         // bytes of a staged row
+  constexpr int CH = SROW / 16;          // 16-byte chunks of a staged row
+  // 16-byte store instructions a wave issues for 32 rows that all exist; they
+  // are the last vector-memory instructions of an item
+  constexpr int kOutStores = 2 * (32 * CH / 64);
+  auto write_out = [&]() __attribute__((always_inline)) {
+    static_assert(4 * 32 * SROW <= TILEB, "four waves stage inside one tile");
+    auto sswz = [](int row) { return SROW == 128 ? ((row >> 1) & 7) : ((row >> 2) & 3); };
+    // Lane coordinates through an opaque copy: the staging and output offsets
+    // below would otherwise be computed once, ahead of the item loop, and sit
+    // in (spilled) registers across the tile loop.
+    int lane_o = lane, lq_o = fr.lq, lh_o = fr.lh;
+    asm volatile("" : "+v"(lane_o), "+v"(lq_o), "+v"(lh_o));
+    const float l_tot = sum_with_other_half(l);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (cur.lp && lh_o == 0 && qrow < len)
+      cur.lp[(int64_t)qrow * p.lse_ss] = l_tot > 0.f ? m + fast_log2(l_tot) : -INFINITY;
+    unsigned char* stage = smem + (wave < 4 ? 0 : VBASE) + (NS - 1) * TILEB + (wave & 3) * 32 * SROW;
 #pragma unroll
-    for (int s0 = 0; s0 < NS - 1; ++s0)
-      if (s0 < n_tiles) {
-        if (s0 == 0) dma_tile(tile_k0(0), ic<0>{});
-        if (s0 == 1) dma_tile(tile_k0(1), ic<1 % NS>{});
-        if (s0 == 2) dma_tile(tile_k0(2), ic<2 % NS>{});
+    for (int ps = 0; ps < 2; ++ps) {
+#pragma unroll
+      for (int dl = 0; dl < DBP; ++dl) {
+        const int db = ps * DBP + dl;
+        if (db < G::NDB) {
+#pragma unroll
+          for (int gq = 0; gq < 4; ++gq) {
+            const int c = 4 * dl + gq;  // chunk of the staged row: columns 8c + 4lh .. +3 of this pass
+            i32x2 w;
+            w[0] = (int)Elem<T>::pack2(O[db][4 * gq] * inv, O[db][4 * gq + 1] * inv);
+            w[1] = (int)Elem<T>::pack2(O[db][4 * gq + 2] * inv, O[db][4 * gq + 3] * inv);
+            *reinterpret_cast<i32x2*>(stage + lq_o * SROW + ((c ^ sswz(lq_o)) << 4) + 8 * lh_o) = w;
+          }
+        }
       }
-    // Everything requested so far must have landed: the Q operands and tile 0
-    // are needed now, and an unconditional full wait here also tells the
-    // compiler that no register load is pending inside the loop (it would
-    // otherwise guard the first use of every Q register there with a wait
-    // that also drains the tile loads).
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int i = 0; i < 32 * CH / 64; ++i) {
+        const int idx = lane_o + 64 * i;
+        const int row = idx / CH, ch = idx % CH;
+        const int och = ps * CH + ch;  // chunk of the output row
+        if (och < G::NCH && q0w + row < len) {
+          const i32x4 val = *reinterpret_cast<const i32x4*>(stage + row * SROW + ((ch ^ sswz(row)) << 4));
+          *reinterpret_cast<i32x4*>(cur.op + (int64_t)(q0w + row) * p.o_ss + och * 8) = val;
+        }
+      }
+      asm volatile("" ::: "memory");
+    }
+  };
+
+  bool have = next_item(cur);
+  if (have) request_item(cur, Qf);
+  int out_stores = 0;  // output stores of the previous item that may still be in flight
+  while (have) {
+    len = cur.len;
+    n_tiles = cur.n_tiles;
+    q0w = cur.q0 + 32 * wave;
+    qrow = q0w + fr.lq;
+    row_lim = causal ? min(qrow, len - 1) : len - 1;  // largest key this lane may see
+    H_w = (len + 31) / 32;                            // halves this wave works on
+    if (causal) H_w = min(H_w, q0w / 32 + 1);         // nothing above its own diagonal block
+    H_w = min(H_w, 2 * n_tiles);
+    if (q0w >= len) H_w = 0;                          // all rows past the sequence end
+#pragma unroll
+    for (int db = 0; db < G::NDB; ++db) O[db] = (f32x16){0};
+    m = -INFINITY;
+    l = 0.f;
+
+    // Every load requested so far must have landed: the Q operands and tile 0
+    // are needed now, and a wait that covers all register loads also tells the
+    // compiler that none is pending inside the loop (it would otherwise guard
+    // the first use of every Q register there with a wait that also drains the
+    // tile loads).  The only younger instructions are the output stores of the
+    // previous item, which may stay in flight: vmcnt retires loads and stores
+    // in issue order, and out_stores is a lower bound of their number.  The
+    // barrier publishes the tiles and separates the previous item's staging
+    // reads from the refill of the last stage, which follows at once.
+    if (out_stores == kOutStores)
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm(kOutStores));
+    else
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __syncthreads();
+    if (NS - 1 < n_tiles) dma.template tile<NS - 1>(cur.kv, (NS - 1) * TN);
     if (H_w > 0) {
       // scores of half 0, its exact row maximum as the first reference point,
       // the probabilities of its first 8 keys, then the first fragments of half 1
@@ -412,117 +712,15 @@ __device__ __forceinline__ void prefill_item(const PrefillParams p, const int bi
         tile_iter(ic<3 % NS>{}, t + 3);
       }
     }
-    __syncthreads();  // the staging below reuses the tile buffers
-  } else {
-  auto step = [&](auto stage_c, int it) {
-    constexpr int ST = decltype(stage_c)::value;
-    // refill the stage that was read in the previous iteration
-    const bool refill = it + NS - 1 < n_tiles;
-    if (refill) dma_tile(tile_k0(it + NS - 1), ic<(ST + NS - 1) % NS>{});
+    __syncthreads();  // every wave is done with the tiles
 
-    const int k0 = tile_k0(it);
-    // whole tile above the diagonal for this wave: nothing to add
-    const bool skip = p.causal && k0 > q0w + 31;
-    if (!skip) {
-      bool need_mask = (k0 + TN > len) || (p.causal && k0 + TN - 1 > q0w);
-      const int wl = p.win_local, wg = p.win_global;
-      if (SPARSE && wl >= 0) need_mask = need_mask || !((k0 + TN - 1 < wg) || (q0w + 31 - k0 < wl));
-      const int causal = p.causal;
-      auto allowed = [&](int key_in_tile) -> bool {
-        const int key = k0 + key_in_tile;
-        bool ok = key < len && (!causal || key <= qrow);
-        if (SPARSE && wl >= 0) ok = ok && ((qrow - key < wl) || (key < wg));
-        return ok;
-      };
-      // V addresses carry VBASE inside the lane offsets (see fr.init)
-      compute_tile<T, D, TN / 32>((uint32_t)(ST * TILEB), (uint32_t)(ST * TILEB), fr, Qf, O, m, l, p.scale, need_mask, allowed);
-    }
-    // The next tile must have landed and everyone must be done with this one.
-    // This wave's loads complete in order, so it is enough that at most the
-    // loads of the NS-2 younger tiles are still in flight (2*IPW each).
-    if (refill)
-      __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * 2 * IPW));
-    else
-      __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-    __syncthreads();
-  };
-
-#pragma unroll
-  for (int s0 = 0; s0 < NS - 1; ++s0)
-    if (s0 < n_tiles) {
-      if (s0 == 0) dma_tile(tile_k0(0), ic<0>{});
-      if (s0 == 1) dma_tile(tile_k0(1), ic<1 % NS>{});
-      if (s0 == 2) dma_tile(tile_k0(2), ic<2 % NS>{});
-    }
-  // tile 0 (and the Q loads issued before it) must be complete
-  if (n_tiles >= NS - 1)
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * 2 * IPW));
-  else
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-  __syncthreads();
-
-  int it = 0;
-  for (; it + NS <= n_tiles; it += NS) {
-    step(ic<0>{}, it);
-    step(ic<1 % NS>{}, it + 1);
-    if (NS > 2) step(ic<2 % NS>{}, it + 2);
-    if (NS > 3) step(ic<3 % NS>{}, it + 3);
-  }
-  if (it < n_tiles) step(ic<0>{}, it++);
-  if (it < n_tiles) step(ic<1 % NS>{}, it++);
-  if (NS > 3 && it < n_tiles) step(ic<2 % NS>{}, it++);
-  }
-
-  // ---- epilogue: normalise, transpose through LDS, coalesced 16-byte stores
-  const float l_tot = sum_with_other_half(l);
-  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  if (p.lse && fr.lh == 0 && qrow < len) {
-    float* lp = p.lse + lse_off + h * p.lse_sh;
-    lp[(int64_t)qrow * p.lse_ss] = l_tot > 0.f ? m + fast_log2(l_tot) : -INFINITY;
-  }
-  unsigned char* stage = smem + wave * 32 * OROWB;
-#pragma unroll
-  for (int db = 0; db < G::NDB; ++db)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int d = 32 * db + 8 * g + 4 * fr.lh;
-      i32x2 w;
-      w[0] = (int)Elem<T>::pack2(O[db][4 * g] * inv, O[db][4 * g + 1] * inv);
-      w[1] = (int)Elem<T>::pack2(O[db][4 * g + 2] * inv, O[db][4 * g + 3] * inv);
-      *reinterpret_cast<i32x2*>(stage + fr.lq * OROWB + d * 2) = w;
-    }
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < (32 * G::NCH + 63) / 64; ++i) {
-    const int idx = lane + 64 * i;
-    const int row = idx / G::NCH, ch = idx % G::NCH;
-    if (((32 * G::NCH) % 64 == 0 || idx < 32 * G::NCH) && q0w + row < len) {
-      const i32x4 val = *reinterpret_cast<const i32x4*>(stage + row * OROWB + ch * 16);
-      *reinterpret_cast<i32x4*>(op + (int64_t)(q0w + row) * p.o_ss + ch * 8) = val;
-    }
-  }
-}
-
-// Persistent launch: the grid holds at most as many workgroups as the device
-// runs at once, and each walks the logical workgroup ids id, id + grid, ...
-// Handing a CU its next q tile this way costs a barrier; a fresh workgroup
-// launch left the CU idle for several microseconds (measured ~12 us between
-// the end of one 512-thread, 128 KiB-LDS workgroup and the first instruction
-// of the next).  Odd rounds are walked back to front within each XCD (id & 7
-// is kept): ids run from the longest q tile of a unit to the shortest, so the
-// workgroup that drew a long tile in one round draws a short one in the next,
-// which balances causal work without a shared counter.
-template <typename T, int D, int NW, int NS, int TN, bool SPARSE>
-__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2)))
-prefill_kernel(const PrefillParams p) {
-  const int grid = gridDim.x;
-  int round = 0;
-  for (int base = 0; base < p.n_items; base += grid, ++round) {
-    int w = blockIdx.x;
-    if ((round & 1) && (grid & 7) == 0) w = (((grid >> 3) - 1 - (w >> 3)) << 3) | (w & 7);
-    const int bid = base + w;
-    if (bid < p.n_items) prefill_item<T, D, NW, NS, TN, SPARSE>(p, bid);
-    if (base + grid < p.n_items) __syncthreads();  // the next item reuses the LDS tiles
+    Item nxt = cur;
+    const bool more = next_item(nxt);
+    if (more) request_item(nxt, Qf);  // (Qf is dead by now; no copy may sit between a load and its wait)
+    write_out();
+    out_stores = (q0w + 32 <= len) ? kOutStores : 0;  // every store instruction had live lanes
+    cur = nxt;
+    have = more;
   }
 }
 
@@ -546,11 +744,16 @@ inline int device_cu_count() {
   return cached[dev] > 0 ? cached[dev] : 0;
 }
 
-template <typename T, int D, int NW, bool SPARSE>
+template <typename T, int D, bool SPARSE>
 int launch_one(const PrefillParams& p, hipStream_t s) {
+  constexpr int NW = (SPARSE ? kSparseRows : kDenseRows) / 32;
   constexpr int NS = SPARSE ? kSparseStages : kDenseStages;
   constexpr int TN = SPARSE ? kSparseTileKeys : kTileN;
-  auto kern = prefill_kernel<T, D, NW, NS, TN, SPARSE>;
+  void (*kern)(const PrefillParams);
+  if constexpr (SPARSE)
+    kern = sparse_kernel<T, D, NW, NS, TN>;
+  else
+    kern = dense_kernel<T, D>;
   constexpr size_t lds = prefill_lds_bytes<D, NW, NS, TN>();
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -571,19 +774,19 @@ int launch_one(const PrefillParams& p, hipStream_t s) {
   return (int)hipGetLastError();
 }
 
-template <int NW, bool SPARSE>
+template <bool SPARSE>
 int dispatch(const PrefillParams& p, int dtype, int head_dim, hipStream_t s) {
   if (dtype == 0) {
     switch (head_dim) {
-      case 64: return launch_one<__bf16, 64, NW, SPARSE>(p, s);
-      case 96: return launch_one<__bf16, 96, NW, SPARSE>(p, s);
-      case 128: return launch_one<__bf16, 128, NW, SPARSE>(p, s);
+      case 64: return launch_one<__bf16, 64, SPARSE>(p, s);
+      case 96: return launch_one<__bf16, 96, SPARSE>(p, s);
+      case 128: return launch_one<__bf16, 128, SPARSE>(p, s);
     }
   } else {
     switch (head_dim) {
-      case 64: return launch_one<_Float16, 64, NW, SPARSE>(p, s);
-      case 96: return launch_one<_Float16, 96, NW, SPARSE>(p, s);
-      case 128: return launch_one<_Float16, 128, NW, SPARSE>(p, s);
+      case 64: return launch_one<_Float16, 64, SPARSE>(p, s);
+      case 96: return launch_one<_Float16, 96, SPARSE>(p, s);
+      case 128: return launch_one<_Float16, 128, SPARSE>(p, s);
     }
   }
   return (int)hipErrorInvalidValue;
@@ -592,10 +795,10 @@ int dispatch(const PrefillParams& p, int dtype, int head_dim, hipStream_t s) {
 }  // namespace
 
 int launch_prefill_dense(const PrefillParams& p, int dtype, int head_dim, hipStream_t s) {
-  return dispatch<kDenseRows / 32, false>(p, dtype, head_dim, s);
+  return dispatch<false>(p, dtype, head_dim, s);
 }
 int launch_prefill_sparse(const PrefillParams& p, int dtype, int head_dim, hipStream_t s) {
-  return dispatch<kSparseRows / 32, true>(p, dtype, head_dim, s);
+  return dispatch<true>(p, dtype, head_dim, s);
 }
 
 }  // namespace mi
