@@ -1,0 +1,86 @@
+"""Compile-time invariants of the dense forward kernel that its hand-counted waits rely on.
+
+The kernel leaves the output stores of a finished work item in flight and waits with
+`s_waitcnt vmcnt(N)` for the loads of the next item; N must not exceed the number of
+store instructions a full wave issues, and the registers that receive the next item's Q
+operands (loaded from inline assembly, invisible to the compiler's own wait insertion)
+must not be copied between the load and that wait.  Both are properties of the generated
+code, so they are checked on the generated code: hipcc cross-compiles without a GPU.
+"""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SRC = os.path.join(ROOT, "tritonops_amd", "csrc", "prefill.hip")
+HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+
+
+@pytest.fixture(scope="module")
+def dense_kernels(tmp_path_factory):
+    if not os.path.exists(HIPCC):
+        pytest.skip("hipcc not available")
+    out = tmp_path_factory.mktemp("asm") / "prefill.s"
+    cmd = [HIPCC, "-x", "hip", "--offload-arch=gfx950", "-O3", "-std=c++17",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-I", os.path.join(ROOT, "include"), "--cuda-device-only", "-S", SRC, "-o", str(out)]
+    subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+    text = out.read_text()
+    kernels = {}
+    for m in re.finditer(r"^(_ZN2mi\S*dense_kernelI(\S+?)Li(\d+)E\S*):", text, re.M):
+        body = text[m.end():text.index("s_endpgm", m.end())]
+        kernels[(m.group(2), int(m.group(3)))] = body.split("\n")
+    assert len(kernels) == 6, sorted(kernels)          # bf16 / f16  x  64 / 96 / 128
+    return kernels
+
+
+def _regs(line):
+    line = line.split(";")[0]
+    found = set()
+    for a, b in re.findall(r"v\[(\d+):(\d+)\]", line):
+        found.update(range(int(a), int(b) + 1))
+    found.update(int(x) for x in re.findall(r"\bv(\d+)\b", line))
+    return found
+
+
+def test_output_store_count_matches_the_counted_wait(dense_kernels):
+    for (dtype, d), lines in dense_kernels.items():
+        stores = [l for l in lines if "global_store_dwordx4" in l]
+        expect = {64: 4, 96: 8, 128: 8}[d]
+        assert len(stores) == expect, (dtype, d, len(stores))
+        waits = {int(x) for l in lines for x in re.findall(r"^\s*s_waitcnt vmcnt\((\d+)\)\s*$", l)}
+        assert expect in waits, (dtype, d, waits)
+
+
+def test_no_scratch_memory(dense_kernels):
+    for key, lines in dense_kernels.items():
+        assert not any("scratch_" in l for l in lines), key
+
+
+def test_q_registers_are_untouched_between_load_and_wait(dense_kernels):
+    for (dtype, d), lines in dense_kernels.items():
+        loads = [(i, l) for i, l in enumerate(lines)
+                 if re.match(r"\s*global_load_dwordx4 v\[\d+:\d+\], v\[\d+:\d+\], off offset:", l)]
+        ksteps = d // 16
+        assert len(loads) == 2 * ksteps, (dtype, d, len(loads))
+        dest = lambda grp: set().union(*[set(range(*map(int, re.search(r"v\[(\d+):(\d+)\]", l).groups()))) |
+                                         {int(re.search(r"v\[(\d+):(\d+)\]", l).group(2))} for _, l in grp])
+        first, second = loads[:ksteps], loads[ksteps:]
+        q = dest(first)
+        assert q == dest(second) and len(q) == 4 * ksteps, (dtype, d)
+        barriers = [i for i, l in enumerate(lines) if "s_barrier" in l]
+        top_barrier = min(i for i in barriers if i > first[-1][0])     # the barrier that opens an item
+        # (a) first item: from its loads to the item's first barrier; (b) later items: from the loads at the
+        # bottom of the item loop to the end of the loop body (it branches back above the same barrier);
+        # (c) from the head of the item loop to that barrier.
+        head = max(i for i, l in enumerate(lines[:top_barrier]) if re.match(r"\.LBB\d+_\d+:.*Loop Header", l))
+        spans = [(first[-1][0] + 1, top_barrier), (second[-1][0] + 1, len(lines)), (head, top_barrier)]
+        for lo, hi in spans:
+            for i in range(lo, hi):
+                l = lines[i]
+                if "global_load_dwordx4" in l and "lds" not in l:
+                    continue
+                assert not (_regs(l) & q), (dtype, d, i, l.strip())
