@@ -74,7 +74,7 @@ void fill_prefill(const A* a, mi::PrefillParams& p, int rows_per_wg) {
   p.lse_sb = a->lse_stride_b; p.lse_ss = a->lse_stride_s; p.lse_sh = a->lse_stride_h;
   p.cu = a->cu_seqlens;
   p.batch = a->batch; p.hq = a->heads_q; p.hkv = a->heads_kv; p.max_seqlen = a->max_seqlen;
-  p.n_qtiles = (a->max_seqlen + rows_per_wg - 1) / rows_per_wg;
+  p.n_qtiles = (int)(((long long)a->max_seqlen + rows_per_wg - 1) / rows_per_wg);
   p.scale = a->scale_log2;
   p.win_local = -1; p.win_global = -1;
 }
@@ -150,8 +150,9 @@ int mi_attn_fwd_validate(const mi_attn_fwd_args* a) {
   if ((rc = check_qkvo(a))) return rc;
   if ((rc = check_prefill_strides(a))) return rc;
   if (a->causal != 0 && a->causal != 1) return fail(MI_ERR_SHAPE, "causal must be 0 or 1");
-  const long long wgs = (long long)((a->max_seqlen + mi::kDenseRows - 1) / mi::kDenseRows) * a->heads_q * a->batch;
-  if (wgs > 0x7fffffffLL) return fail(MI_ERR_SHAPE, "grid of %lld workgroups is too large", wgs);
+  // (work item ids are 32-bit and the persistent kernel steps them by its grid size)
+  const long long wgs = (((long long)a->max_seqlen + mi::kDenseRows - 1) / mi::kDenseRows) * a->heads_q * a->batch;
+  if (wgs > 0x3fffffffLL) return fail(MI_ERR_SHAPE, "%lld work items are too many", wgs);
   return MI_OK;
 }
 
@@ -411,7 +412,7 @@ int mi_attn_fwd_blocksparse_validate(const mi_attn_sparse_args* a) {
     return fail(MI_ERR_SPARSE_LAYOUT, "mask strides must be >= 0");
   if ((a->window_local < 0) != (a->window_global < 0) || a->window_local < -1 || a->window_global < -1)
     return fail(MI_ERR_SPARSE_LAYOUT, "window_local/window_global must both be -1 or both be >= 0");
-  const long long wgs = (long long)((a->max_seqlen + mi::kSparseRows - 1) / mi::kSparseRows) * a->heads_q * a->batch;
+  const long long wgs = (((long long)a->max_seqlen + mi::kSparseRows - 1) / mi::kSparseRows) * a->heads_q * a->batch;
   if (wgs > 0x7fffffffLL) return fail(MI_ERR_SHAPE, "grid of %lld workgroups is too large", wgs);
   return MI_OK;
 }
