@@ -212,3 +212,25 @@ def test_long_ragged_batch_with_many_tiles():
     nc = ta.flash_attention(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), causal=False)
     want_nc = orc.varlen_masked_attention(q, k, v, cu, lambda L: torch.ones(L, L, dtype=torch.bool), faithful=False)
     assert_close(nc, want_nc, TOL)
+
+
+@pytest.mark.parametrize("D,dtype", [(64, torch.float16), (96, torch.bfloat16), (128, torch.float16)])
+def test_many_work_items_per_workgroup(D, dtype):
+    """A packed batch whose q tiles outnumber the CUs several times over, with
+    empty sequences, sequences of one token and q tiles that do not exist for
+    the shorter sequences: every workgroup walks a dozen work items, skips
+    some, and overlaps the write-out of one with the loads of the next."""
+    import tritonops_amd as ta
+
+    lens = torch.tensor([0, 1, 300, 257, 2049, 511, 0, 1500, 31, 1024, 513, 2500, 255, 256, 1000, 2047, 64, 700, 1,
+                         1280], dtype=torch.int32)
+    cu = cu_from(lens)
+    T = int(cu[-1])
+    Hq, Hkv = 16, 4
+    q, k, v = randn((1, T, Hq, D), 4, dtype), randn((1, T, Hkv, D), 5, dtype), randn((1, T, Hkv, D), 6, dtype)
+    want, want_lse = orc.flash_attn_torch(q, k, v, cu, faithful=False, return_lse=True)
+    got, lse = ta.flash_attn_triton_fwd(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), D ** -0.5 * ta.LOG2E)
+    assert_close(got, want, TOL)
+    _lse_close(lse, want_lse)
+    again, lse2 = ta.flash_attn_triton_fwd(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), D ** -0.5 * ta.LOG2E)
+    assert torch.equal(again, got) and torch.equal(lse2, lse)
