@@ -92,8 +92,7 @@ extern __shared__ __attribute__((aligned(1024))) unsigned char smem_bwd[];
 constexpr int kBwdStages = 3;  // streamed tile pairs resident in LDS (4 measured the same)
 
 template <typename T, int D, int MODE>
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2)))
-bwd_kernel(const BwdParams p) {
+__device__ __forceinline__ void bwd_item(const BwdParams& p, const int bid) {
   using G = RowGeom<D>;
   using F = UniFrags<D>;
   constexpr int NW = 8, BM = 32 * NW, TN = 64, NS = kBwdStages;
@@ -106,7 +105,11 @@ bwd_kernel(const BwdParams p) {
   constexpr int OROWB = D * 2 + 16;               // epilogue staging row
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63;
+  int lane = tid & 63;
+  // An opaque copy per item: what is derived from the lane id (fragment
+  // addresses, load offsets) is then recomputed for every item instead of
+  // being held in registers across the whole item loop, where it was spilled.
+  asm volatile("" : "+v"(lane));
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
   const int heads_r = MODE == kDQ ? p.hq : p.hkv;
@@ -119,7 +122,6 @@ bwd_kernel(const BwdParams p) {
   const int n_units = p.batch * heads_r;
   int unit, slot;
   {
-    const int bid = blockIdx.x;
     if ((n_units & 7) == 0) {
       const int sl = bid >> 3;
       unit = (sl / p.n_rtiles) * 8 + (bid & 7);
@@ -453,6 +455,25 @@ bwd_kernel(const BwdParams p) {
   }
 }
 
+// Persistent launch, as in the forward pass: at most one workgroup per CU, each
+// walking the work item ids id, id + grid, ... (a fresh 512-thread workgroup
+// with this much LDS starts several microseconds after its predecessor ends);
+// odd rounds run back to front within an XCD so that a workgroup that drew an
+// item that streams many tiles draws one that streams few next.
+template <typename T, int D, int MODE>
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2)))
+bwd_kernel(const BwdParams p, const int n_items) {
+  const int grid = gridDim.x;
+  int round = 0;
+  for (int base = 0; base < n_items; base += grid, ++round) {
+    int w = blockIdx.x;
+    if ((round & 1) && (grid & 7) == 0) w = (((grid >> 3) - 1 - (w >> 3)) << 3) | (w & 7);
+    const int bid = base + w;
+    if (bid < n_items) bwd_item<T, D, MODE>(p, bid);
+    if (base + grid < n_items) __syncthreads();  // the next item's tiles overwrite the staging area
+  }
+}
+
 // Delta[b][h][s] = sum_d o[s][d] * do[s][d], fp32.  16 lanes per row (one 16-byte
 // chunk each), 16 rows per 256-thread workgroup.
 template <typename T>
@@ -493,8 +514,11 @@ int launch_mode(const BwdParams& p, hipStream_t s) {
   auto kern = bwd_kernel<T, D, MODE>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return (int)e;
-  const long long grid = (long long)p.n_rtiles * (MODE == kDQ ? p.hq : p.hkv) * p.batch;
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, s, p);
+  const long long items = (long long)p.n_rtiles * (MODE == kDQ ? p.hq : p.hkv) * p.batch;
+  long long grid = items;
+  const int cus = device_cu_count();
+  if (cus > 0 && grid > cus) grid = cus;  // one workgroup per CU is resident (LDS)
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, s, p, (int)items);
   return (int)hipGetLastError();
 }
 

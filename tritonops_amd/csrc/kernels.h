@@ -120,6 +120,9 @@ struct XentGradParams {
   int32_t vec;         // rows can be accessed in 16-byte chunks
 };
 
+// CUs of the current device (cached per device; 0 if the query fails).
+int device_cu_count();
+
 // dtype: 0 bf16, 1 f16.  head_dim in {64, 96, 128}.  Return hipError_t as int.
 int launch_prefill_dense(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);
 int launch_prefill_sparse(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);

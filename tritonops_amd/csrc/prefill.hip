@@ -731,19 +731,6 @@ constexpr size_t prefill_lds_bytes() {
   return pipe > epi ? pipe : epi;
 }
 
-// CUs of the current device (cached per device; 0 if the query fails)
-inline int device_cu_count() {
-  static int cached[64] = {0};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-  if (cached[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
-    cached[dev] = n > 0 ? n : -1;
-  }
-  return cached[dev] > 0 ? cached[dev] : 0;
-}
-
 template <typename T, int D, bool SPARSE>
 int launch_one(const PrefillParams& p, hipStream_t s) {
   constexpr int NW = (SPARSE ? kSparseRows : kDenseRows) / 32;
@@ -793,6 +780,19 @@ int dispatch(const PrefillParams& p, int dtype, int head_dim, hipStream_t s) {
 }
 
 }  // namespace
+
+// CUs of the current device (cached per device; 0 if the query fails)
+int device_cu_count() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+    cached[dev] = n > 0 ? n : -1;
+  }
+  return cached[dev] > 0 ? cached[dev] : 0;
+}
 
 int launch_prefill_dense(const PrefillParams& p, int dtype, int head_dim, hipStream_t s) {
   return dispatch<false>(p, dtype, head_dim, s);
