@@ -309,6 +309,11 @@ __device__ __forceinline__ void bwd_item(const BwdParams& p, const int bid) {
 #pragma unroll
         for (int st = 0; st < kPrefetch; ++st) f[st] = frag(st);
       }
+      // Issue priority: highest while the wave feeds the accumulators (the last
+      // product, 2*NDB MFMAs over NDB independent chains), low during the two
+      // serial chains S and dP; the two waves of a SIMD then fall out of step
+      // instead of competing with the same kind of work (measured 3 %).
+      __builtin_amdgcn_s_setprio(1);
 #pragma unroll
       for (int st = 0; st < G::KSTEPS; ++st) {
         S = Elem<T>::mfma(f[st % kPrefetch], Xf[st], S);
@@ -356,6 +361,7 @@ __device__ __forceinline__ void bwd_item(const BwdParams& p, const int bid) {
       __builtin_amdgcn_sched_barrier(0);
       // last product: 2*NDB MFMAs, fragment (kk, db) = step kk*NDB + db
       constexpr int NACC = 2 * G::NDB;
+      __builtin_amdgcn_s_setprio(3);
 #pragma unroll
       for (int i = 0; i < NACC; ++i) {
         const int kk = i / G::NDB, db = i % G::NDB;
@@ -416,6 +422,7 @@ __device__ __forceinline__ void bwd_item(const BwdParams& p, const int bid) {
       step(ic<3 % NS>{}, u + 3);
     }
   }
+  __builtin_amdgcn_s_setprio(0);
   __syncthreads();
 
   // ---- epilogue: scale, transpose through LDS, coalesced 16-byte stores

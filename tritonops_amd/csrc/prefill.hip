@@ -534,6 +534,11 @@ dense_kernel(const PrefillParams p) {
     uint32_t (&Pc)[8] = Pb[KB];
     uint32_t (&Pn)[8] = Pb[KB ^ 1];
     const float m_neg = (m == -INFINITY) ? 0.f : -m;
+    // Block A carries the serial chain of the eight S MFMAs: a raised issue
+    // priority while a wave is in it (and a lower one in block B, whose MFMAs
+    // form four independent chains) lets the two waves of a SIMD fall out of
+    // step, one in A while the other is in B; measured 1 % on the launch.
+    __builtin_amdgcn_s_setprio(3);
     i32x4 vf[G::NDB];
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
@@ -556,6 +561,7 @@ dense_kernel(const PrefillParams p) {
     l += rsv[KB];
     mask_half(h + 1, Sn);
     const float m_neg2 = (m == -INFINITY) ? 0.f : -m;
+    __builtin_amdgcn_s_setprio(1);
     rsv[KB ^ 1] = 0.f;
 #pragma unroll
     for (int sl = 0; sl < 8; ++sl) {
@@ -712,6 +718,7 @@ dense_kernel(const PrefillParams p) {
         tile_iter(ic<3 % NS>{}, t + 3);
       }
     }
+    __builtin_amdgcn_s_setprio(0);
     __syncthreads();  // every wave is done with the tiles
 
     Item nxt = cur;
