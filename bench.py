@@ -62,12 +62,17 @@ def _time_steps(fn, steps, warmup):
 
 
 def _event_ms(kind, args, steps, warmup):
-    """Average launch duration from HIP events on the current stream."""
+    """Average launch duration from HIP events on the current stream.  `args` is
+    one argument struct or a list of them (launch i uses struct i % len)."""
     from tritonops_amd import _lib
     lib = _lib.load()
     ms = C.c_float(0)
     st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    _lib.check(lib.mi_time_launches(kind, C.cast(C.byref(args), C.c_void_p), st, warmup, steps, C.byref(ms)))
+    if not isinstance(args, (list, tuple)):
+        args = [args]
+    arr = (type(args[0]) * len(args))(*args)
+    _lib.check(lib.mi_time_launches(kind, C.cast(arr, C.c_void_p), len(args), C.sizeof(args[0]), st, warmup, steps,
+                                    C.byref(ms)))
     return ms.value
 
 
@@ -124,7 +129,7 @@ def run_dense_bwd(steps, warmup):
     sm = D ** -0.5 * ta.LOG2E
     o, lse = ops._dense_fwd(qs, ks, vs, None, sm, True, None, bhsd=True)
     steps, warmup = max(4, steps // 4), max(2, warmup // 4)         # a step is ~5x the forward
-    fn = lambda: ops._dense_bwd(qs, ks, vs, o, lse, ds, None, sm, True, None)
+    fn = lambda: ops._dense_bwd(qs, ks, vs, o, ds, lse, None, sm, True, None)
     ms = _time_steps(fn, steps, warmup)
     dq, dk, dv = fn()
     a = _lib.AttnBwdArgs()

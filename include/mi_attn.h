@@ -16,7 +16,8 @@
  *   - the innermost (head_dim) axis of q/k/v/o must be contiguous and every
  *     row must start on a 16-byte boundary (strides are in ELEMENTS);
  *   - return value: MI_OK (0) or a negative mi_status; nothing throws, nothing
- *     allocates or frees device memory, nothing synchronises the device;
+ *     allocates or frees device memory, nothing synchronises the device (the
+ *     blocking timing helper for benchmarks lives in mi_attn_bench.h);
  *   - all argument validation happens on the host before any HIP call, so it
  *     can be exercised on a machine without a GPU;
  *   - log-sum-exp values are base 2 of the scaled scores, fp32:
@@ -35,7 +36,7 @@
 extern "C" {
 #endif
 
-#define MI_ATTN_ABI_VERSION 4
+#define MI_ATTN_ABI_VERSION 5
 
 /* KV tile edge (tokens) of the prefill kernels and block edge of the block
  * sparse layouts; fixed at build time. */
@@ -410,22 +411,15 @@ int mi_abi_version(void);
 const char *mi_last_error(void);
 /* Name of a status code. */
 const char *mi_status_name(int status);
+/* Compute units of the current HIP device, the figure the library's own
+ * launches and the mi_decode_choose_* heuristics are sized with (0 when no
+ * device can be queried; the heuristics then assume 256). */
+int mi_device_cu_count(void);
 /* Validate without launching (what the launch entry points run first). */
 int mi_attn_fwd_validate(const mi_attn_fwd_args *args);
 int mi_attn_fwd_blocksparse_validate(const mi_attn_sparse_args *args);
 int mi_decode_validate(const mi_decode_args *args);
 int mi_attn_bwd_validate(const mi_attn_bwd_args *args);
-
-/* Average device time per launch, measured with HIP events on `stream` around
- * `iters` back-to-back launches of the given entry point (after `warmup`
- * untimed ones).  Blocks the calling thread; for benchmarking only.
- * kind: 0 = mi_attn_fwd, 1 = mi_attn_fwd_blocksparse, 2 = mi_decode,
- *       3 = mi_decode_splitkv, 4 = mi_decode_merge, 5 = mi_attn_bwd,
- *       6 = mi_rmsnorm_fwd, 7 = mi_rmsnorm_bwd, 8 = mi_xent_fwd,
- *       9 = mi_xent_dlogits, 10 = mi_xent_bwd_dlogits.
- * Returns MI_OK and writes milliseconds to *ms_per_launch. */
-int mi_time_launches(int kind, const void *args, void *stream, int warmup,
-                     int iters, float *ms_per_launch);
 
 #ifdef __cplusplus
 }

@@ -11,7 +11,7 @@ import pytest
 from tritonops_amd import _lib
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "mi_attn.h")
+HEADERS = [os.path.join(ROOT, "include", n) for n in ("mi_attn.h", "mi_attn_bench.h")]
 
 
 @pytest.fixture(scope="module")
@@ -20,14 +20,14 @@ def lib():
 
 
 def test_every_declared_symbol_is_exported(lib):
-    text = open(HEADER).read()
+    text = "".join(open(h).read() for h in HEADERS)
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     declared = set(re.findall(r"\b(mi_[a-z_0-9]+)\s*\(", text))
     assert declared, "no prototypes found in the header"
     assert declared == set(_lib.EXPORTS), "ctypes table and header disagree: %s" % (declared ^ set(_lib.EXPORTS))
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.mi_abi_version() == _lib.MI_ATTN_ABI_VERSION == 4
+    assert lib.mi_abi_version() == _lib.MI_ATTN_ABI_VERSION == 5
 
 
 def test_struct_layout_matches_the_c_compiler(tmp_path):
@@ -168,6 +168,9 @@ def test_decode_geometry_and_validation(lib):
         (lambda a: setattr(a, "heads_kv", 0), "MI_ERR_GQA"),
         (lambda a: (setattr(a, "heads_q", 66), setattr(a, "heads_kv", 2)), "MI_ERR_GQA"),   # 33 per kv head
         (lambda a: setattr(a, "k_stride_s", 12), "MI_ERR_STRIDE"),
+        # a tile is addressed with 32-bit byte offsets: negative or huge row strides would wrap
+        (lambda a: setattr(a, "k_stride_s", -128), "MI_ERR_STRIDE"),
+        (lambda a: setattr(a, "v_stride_s", 1 << 24), "MI_ERR_STRIDE"),
         (lambda a: setattr(a, "head_dim", 32), "MI_ERR_HEAD_DIM"),
     ]:
         a = _good_decode()
@@ -175,6 +178,9 @@ def test_decode_geometry_and_validation(lib):
         rc = lib.mi_decode_validate(C.byref(a))
         assert lib.mi_status_name(rc).decode() == want, (want, rc, _err(lib))
         assert lib.mi_decode(C.byref(a), None) == rc
+    a = _good_decode()
+    a.k_stride_s = a.v_stride_s = (1 << 24) - 8
+    assert lib.mi_decode_validate(C.byref(a)) == 0
     # sparse form
     a = _good_decode()
     a.block_idx = 0x5000
@@ -183,6 +189,14 @@ def test_decode_geometry_and_validation(lib):
     assert lib.mi_decode_num_splits(C.byref(a)) == 17
     assert lib.mi_decode_validate(C.byref(a)) == 0
     a.block_size = 32
+    assert lib.mi_status_name(lib.mi_decode_validate(C.byref(a))).decode() == "MI_ERR_SPARSE_LAYOUT"
+    # an empty list is valid exactly when the implicit last block is attended
+    a.block_size, a.max_blocks, a.include_last_block = 64, 0, 1
+    assert lib.mi_decode_validate(C.byref(a)) == 0 and lib.mi_decode_num_splits(C.byref(a)) == 1
+    a.include_last_block = 0
+    assert lib.mi_status_name(lib.mi_decode_validate(C.byref(a))).decode() == "MI_ERR_SPARSE_LAYOUT"
+    a.max_blocks = -1
+    a.include_last_block = 1
     assert lib.mi_status_name(lib.mi_decode_validate(C.byref(a))).decode() == "MI_ERR_SPARSE_LAYOUT"
 
 
@@ -326,11 +340,12 @@ def test_split_blocks_heuristic(lib):
 
 def test_time_launches_rejects_bad_arguments(lib):
     ms = C.c_float()
-    assert lib.mi_time_launches(0, None, None, 0, 1, C.byref(ms)) == -1
+    assert lib.mi_time_launches(0, None, 1, 0, None, 0, 1, C.byref(ms)) == -6
     a = _good_fwd()
-    assert lib.mi_time_launches(11, C.cast(C.byref(a), C.c_void_p), None, 0, 1, C.byref(ms)) == -6
+    assert lib.mi_time_launches(12, C.cast(C.byref(a), C.c_void_p), 1, 0, None, 0, 1, C.byref(ms)) == -6
+    assert lib.mi_time_launches(0, C.cast(C.byref(a), C.c_void_p), 0, 0, None, 0, 1, C.byref(ms)) == -6
     a.head_dim = 5
-    assert lib.mi_time_launches(0, C.cast(C.byref(a), C.c_void_p), None, 1, 1, C.byref(ms)) == -4
+    assert lib.mi_time_launches(0, C.cast(C.byref(a), C.c_void_p), 1, 0, None, 1, 1, C.byref(ms)) == -4
 
 
 def test_python_wrappers_refuse_cpu_tensors():
@@ -343,7 +358,74 @@ def test_python_wrappers_refuse_cpu_tensors():
     with pytest.raises(RuntimeError, match="GPU only"):
         ta.flash_attention(q, q, q, cu)
     with pytest.raises(RuntimeError, match="GPU only"):
-        ta.flash_attention_decoding(q[0], q, q, cu)
+        ta.flash_attention_decoding(q[:, 0], q, q, cu)
+
+
+def test_python_wrappers_check_extents_before_any_launch():
+    """The kernels take every extent from q: a shorter k / v, a mis-shaped do or
+    lse, or a wrong index tensor must be refused on the host (no GPU needed)."""
+    import torch
+
+    import tritonops_amd as ta
+    from tritonops_amd import ops
+
+    bf = torch.bfloat16
+    q = torch.zeros(1, 16, 4, 64, dtype=bf)
+    k = torch.zeros(1, 16, 2, 64, dtype=bf)
+    cu = torch.tensor([0, 16], dtype=torch.int32)
+    lse = torch.zeros(1, 16, 4)
+    for bad_k, bad_v in ((k[:, :8], k), (k, k[:, :8]), (k, k[:, :, :1]), (k.float(), k), (k[..., :32], k[..., :32]),
+                         (torch.zeros(1, 16, 3, 64, dtype=bf),) * 2):
+        with pytest.raises(ValueError):
+            ta.flash_attention(q, bad_k, bad_v, cu)
+        with pytest.raises(ValueError):
+            ta.flash_attn_sparse_triton(q, bad_k, bad_v, cu, None, 64, 64)
+        with pytest.raises(ValueError):
+            ta.flash_attn_triton_bwd(q, bad_k, bad_v, q, q, lse, cu, 0.1)
+    with pytest.raises(ValueError):                      # batched form: [B, H, S, D]
+        ta.flash_attention(q.transpose(1, 2), k.transpose(1, 2)[:, :, :8], k.transpose(1, 2)[:, :, :8])
+    for o, do, l in ((q[:, :8], q, lse), (q, q[:, :8], lse), (q, q, lse[:, :8]), (q, q, lse.double()),
+                     (q, q.float(), lse), (q, lse, q)):     # the last one: do and lse swapped
+        with pytest.raises(ValueError):
+            ta.flash_attn_triton_bwd(q, k, k, o, do, l, cu, 0.1)
+    # all extents right: the call gets as far as the device check
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ta.flash_attn_triton_bwd(q, k, k, q, q, lse, cu, 0.1)
+
+    qd = torch.zeros(2, 4, 64, dtype=bf)
+    kd = torch.zeros(2, 128, 2, 64, dtype=bf)
+    cu2 = torch.tensor([0, 100, 228], dtype=torch.int32)
+    with pytest.raises(ValueError):
+        ta.flash_attention_decoding(qd, kd, kd[:, :64], cu2)
+    with pytest.raises(ValueError):
+        ta.flash_attention_decoding(qd, kd, kd.half(), cu2)
+    with pytest.raises(ValueError):
+        ta.flash_attention_decoding(qd, kd, kd, cu2[:2])
+    with pytest.raises(ValueError):
+        ta.flash_attention_decoding(qd, kd, kd, None, seq_lens=torch.tensor([1.0, 2.0]))
+    with pytest.raises(ValueError):
+        ta.flash_attention_decoding(qd, kd, kd, cu2, kv_layout="paged", page_table=torch.zeros(2, 2), page_size=128)
+    for idx in (torch.zeros(2, 2, 3), torch.zeros(2, 3, dtype=torch.int32), torch.zeros(1, 2, 3, dtype=torch.int32)):
+        with pytest.raises(ValueError):
+            ta.flash_attention_sparse_decoding(qd, kd, kd, cu2, block_indices=idx)
+    with pytest.raises(ValueError):
+        ta.flash_attention_sparse_decoding(qd, kd, kd, cu2, block_indices=torch.zeros(2, 2, 1, dtype=torch.int32),
+                                           block_counts=torch.zeros(2, 3, dtype=torch.int32))
+    with pytest.raises(ValueError):
+        ta.flash_attention_sparse_decoding(qd, kd, kd, cu2, block_indices=torch.zeros(2, 2, 0, dtype=torch.int32),
+                                           include_last_block=False)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ta.flash_attention_decoding(qd, kd, kd, cu2)
+
+
+def test_window_csr_is_built_once():
+    from tritonops_amd import masks
+
+    a = masks.window_csr(40, 200, 128, "cpu")
+    b = masks.window_csr(40, 200, 128, "cpu")
+    assert a[0] is b[0] and a[1] is b[1]
+    want = masks.block_mask_to_csr(masks.window_block_mask(40, 200, 128), "cpu")
+    assert (a[0] == want[0]).all() and (a[1] == want[1]).all() and a[2] == want[2]
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

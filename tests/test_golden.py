@@ -124,7 +124,7 @@ def test_gpu_matches_neighbour_fixtures(nb):
     d = lambda t: t.cuda()
     c = nb["attn_backward"]
     o, lse = ta.flash_attn_triton_fwd(d(c["q"]), d(c["k"]), d(c["v"]), d(c["cu"]), 64 ** -0.5 * ta.LOG2E)
-    dq, dk, dv = ta.flash_attn_triton_bwd(d(c["q"]), d(c["k"]), d(c["v"]), o, lse, d(c["do"]), d(c["cu"]),
+    dq, dk, dv = ta.flash_attn_triton_bwd(d(c["q"]), d(c["k"]), d(c["v"]), o, d(c["do"]), lse, d(c["cu"]),
                                           64 ** -0.5 * ta.LOG2E)
     for name, g in (("dq", dq), ("dk", dk), ("dv", dv)):
         assert_close(g, c[name], 3e-2 * max(1.0, c[name].abs().max().item()), name)

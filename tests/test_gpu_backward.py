@@ -44,7 +44,7 @@ def test_packed_causal_backward_matches_oracle(lens, Hq, Hkv, D, dtype):
     wq, wk, wv = orc.varlen_masked_attention_backward(q, k, v, do, cu, orc.causal_mask)
     sm = D ** -0.5 * ta.LOG2E
     o, lse = ta.flash_attn_triton_fwd(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), sm)
-    dq, dk, dv = ta.flash_attn_triton_bwd(q.cuda(), k.cuda(), v.cuda(), o, lse, do.cuda(), cu.cuda(), sm)
+    dq, dk, dv = ta.flash_attn_triton_bwd(q.cuda(), k.cuda(), v.cuda(), o, do.cuda(), lse, cu.cuda(), sm)
     assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape and dq.dtype == dtype
     _check(dq, wq, "dq")
     _check(dk, wk, "dk")
@@ -85,7 +85,7 @@ def test_batched_backward_through_the_c_abi(causal):
     sm = D ** -0.5 * ta.LOG2E
     qc, kc, vc, dc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
     o, lse = ops._dense_fwd(qc, kc, vc, None, sm, causal, None)
-    dq, dk, dv = ops._dense_bwd(qc, kc, vc, o, lse, dc, None, sm, causal, None)
+    dq, dk, dv = ops._dense_bwd(qc, kc, vc, o, dc, lse, None, sm, causal, None)
     mask = orc.causal_mask if causal else (lambda L: torch.ones(L, L, dtype=torch.bool))
     for b in range(B):
         cu = torch.tensor([0, S], dtype=torch.int32)

@@ -271,3 +271,20 @@ def test_large_ragged_batch_is_dealt_to_the_resident_waves(split_tokens):
     assert_close(got, want, TOL, "o")
     assert torch.count_nonzero(got[::7]) == 0
     assert torch.isinf(lse[::7]).all() and torch.isfinite(lse[lens.cuda() > 0]).all()
+
+
+def test_empty_block_list_attends_the_last_block_only():
+    """block_indices [B, Hkv, 0] with include_last_block: the list is empty and
+    the block holding the newest token is the only one attended."""
+    import tritonops_amd as ta
+
+    B, Hq, Hkv, D, L = 3, 4, 2, 128, 300
+    lens = torch.tensor([300, 64, 0], dtype=torch.int32)
+    q = randn((B, Hq, D), 1)
+    k, v = _kv(B, L, Hkv, D, torch.bfloat16, 2)
+    idx = torch.zeros((B, Hkv, 0), dtype=torch.int32)
+    want = orc.block_sparse_decoding(q, k, v, lens, idx, include_last_block=True, faithful=False)
+    got = ta.flash_attention_sparse_decoding(q.cuda(), k.cuda(), v.cuda(), None, seq_lens=lens.cuda(),
+                                             block_indices=idx.cuda())
+    assert_close(got, want, TOL)
+    assert torch.count_nonzero(got[2]) == 0

@@ -80,7 +80,7 @@ def test_packed_forward_and_backward_replay_like_eager():
 
     def run():
         o, lse = ta.flash_attn_triton_fwd(q, k, v, cu, sm, max_seq_len=max(lens))
-        dq, dk, dv = ta.flash_attn_triton_bwd(q, k, v, o, lse, do, cu, sm, max_seq_len=max(lens))
+        dq, dk, dv = ta.flash_attn_triton_bwd(q, k, v, o, do, lse, cu, sm, max_seq_len=max(lens))
         return o, lse, dq, dk, dv
 
     for i, t in enumerate(inputs):

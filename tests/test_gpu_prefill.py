@@ -234,3 +234,23 @@ def test_many_work_items_per_workgroup(D, dtype):
     _lse_close(lse, want_lse)
     again, lse2 = ta.flash_attn_triton_fwd(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), D ** -0.5 * ta.LOG2E)
     assert torch.equal(again, got) and torch.equal(lse2, lse)
+
+
+def test_rows_outside_every_sequence_are_zero():
+    """Packed buffers longer than cu_seq_lens[-1]: rows that belong to no
+    sequence come back as zeros in o and lse, as from the reference's
+    zero-filled outputs (flash_attn_triton.py:608-609)."""
+    import tritonops_amd as ta
+
+    lens = torch.tensor([70, 130], dtype=torch.int32)
+    cu = cu_from(lens)
+    T, pad, Hq, Hkv, D = int(cu[-1]), 56, 4, 2, 128
+    q, k, v = randn((1, T + pad, Hq, D), 1), randn((1, T + pad, Hkv, D), 2), randn((1, T + pad, Hkv, D), 3)
+    sm = D ** -0.5 * ta.LOG2E
+    o, lse = ta.flash_attn_triton_fwd(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), sm)
+    want, want_lse = orc.flash_attn_torch(q[:, :T], k[:, :T], v[:, :T], cu, faithful=False, return_lse=True)
+    assert_close(o[:, :T], want, TOL)
+    assert (lse[:, :T].cpu() - want_lse).abs().max() <= LSE_TOL
+    assert torch.count_nonzero(o[:, T:]) == 0 and torch.count_nonzero(lse[:, T:]) == 0
+    so, slse = ta.flash_attn_sparse_triton(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), None, 64, 64)
+    assert torch.count_nonzero(so[:, T:]) == 0 and torch.count_nonzero(slse[:, T:]) == 0

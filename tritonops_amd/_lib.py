@@ -9,7 +9,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmi_attn.so")
 
-MI_ATTN_ABI_VERSION = 4
+MI_ATTN_ABI_VERSION = 5
 MI_KV_BATCHED, MI_KV_PACKED, MI_KV_PAGED = 0, 1, 2
 MI_ATTN_BLOCK = 64
 MI_DTYPE_F32 = 2
@@ -178,7 +178,9 @@ EXPORTS = {
     "mi_attn_fwd_validate": (C.c_int, [C.POINTER(AttnFwdArgs)]),
     "mi_attn_fwd_blocksparse_validate": (C.c_int, [C.POINTER(AttnSparseArgs)]),
     "mi_decode_validate": (C.c_int, [C.POINTER(DecodeArgs)]),
-    "mi_time_launches": (C.c_int, [C.c_int, _vp, _vp, C.c_int, C.c_int, C.POINTER(C.c_float)]),
+    "mi_device_cu_count": (C.c_int, []),
+    # include/mi_attn_bench.h
+    "mi_time_launches": (C.c_int, [C.c_int, _vp, C.c_int, _sz, _vp, C.c_int, C.c_int, C.POINTER(C.c_float)]),
 }
 
 

@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(HERE, "libmi_attn.so")
-SOURCES = ["api.cpp", "prefill.hip", "decode.hip", "bwd.hip", "rmsnorm.hip", "xent.hip"]
+SOURCES = ["api.cpp", "bench_timing.cpp", "prefill.hip", "decode.hip", "bwd.hip", "rmsnorm.hip", "xent.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950",

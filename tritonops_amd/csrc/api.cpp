@@ -443,8 +443,10 @@ static int decode_validate_shape(const mi_decode_args* a) {
     if (a->block_size != MI_ATTN_BLOCK) return fail(MI_ERR_SPARSE_LAYOUT, "block_size %d must be %d", a->block_size, MI_ATTN_BLOCK);
     if (a->include_last_block != 0 && a->include_last_block != 1)
       return fail(MI_ERR_SPARSE_LAYOUT, "include_last_block must be 0 or 1");
-    if (a->max_blocks <= 0 || a->split_blocks <= 0)
-      return fail(MI_ERR_SPARSE_LAYOUT, "max_blocks %d and split_blocks %d must be positive", a->max_blocks, a->split_blocks);
+    // an empty list is a valid one when the implicit last block is attended
+    if (a->max_blocks < 0 || a->max_blocks + a->include_last_block <= 0 || a->split_blocks <= 0)
+      return fail(MI_ERR_SPARSE_LAYOUT, "max_blocks %d (+ the implicit last block) and split_blocks %d must be positive",
+                  a->max_blocks, a->split_blocks);
     if (a->block_idx_stride_b < 0 || a->block_idx_stride_h < 0)
       return fail(MI_ERR_SPARSE_LAYOUT, "block_idx strides must be >= 0");
     if ((a->window_local < 0) != (a->window_global < 0) || a->window_local < -1 || a->window_global < -1)
@@ -503,7 +505,8 @@ int mi_decode_choose_split_blocks(int batch, int heads_kv, int total_blocks, int
   return (int)((total_blocks + chunks - 1) / chunks);
 }
 
-int mi_decode_validate(const mi_decode_args* a) {
+// everything but the workspace
+static int decode_validate_args(const mi_decode_args* a) {
   int rc = decode_validate_shape(a);
   if (rc) return rc;
   if (!a->q || !a->k || !a->v || !a->o) return fail(MI_ERR_NULL_POINTER, "q, k, v and o must be non-NULL");
@@ -519,6 +522,16 @@ int mi_decode_validate(const mi_decode_args* a) {
                        a->v_stride_b, a->v_stride_s, a->v_stride_h};
   for (int64_t x : s)
     if (!mult8(x)) return fail(MI_ERR_STRIDE, "q/k/v strides must be multiples of 8 elements (got %lld)", (long long)x);
+  // a 32-key tile is addressed as scalar base + 32-bit byte offset per lane
+  if (a->k_stride_s < 0 || a->v_stride_s < 0 || a->k_stride_s >= (1 << 24) || a->v_stride_s >= (1 << 24))
+    return fail(MI_ERR_STRIDE, "k/v sequence strides must be in [0, 2^24) elements (got %lld, %lld)",
+                (long long)a->k_stride_s, (long long)a->v_stride_s);
+  return MI_OK;
+}
+
+int mi_decode_validate(const mi_decode_args* a) {
+  int rc = decode_validate_args(a);
+  if (rc) return rc;
   if (!a->workspace) return fail(MI_ERR_NULL_POINTER, "workspace is NULL");
   if (!aligned16(a->workspace)) return fail(MI_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
   const size_t need = mi_decode_workspace_bytes(a);
@@ -551,45 +564,6 @@ int mi_decode(const mi_decode_args* a, void* stream) {
   return mi_decode_merge(a, stream);
 }
 
-int mi_time_launches(int kind, const void* args, void* stream, int warmup, int iters, float* ms_per_launch) {
-  if (!args || !ms_per_launch) return fail(MI_ERR_NULL_POINTER, "args / ms_per_launch is NULL");
-  if (iters <= 0 || warmup < 0 || kind < 0 || kind > 10) return fail(MI_ERR_SHAPE, "bad kind / warmup / iters");
-  auto once = [&]() -> int {
-    switch (kind) {
-      case 0: return mi_attn_fwd(static_cast<const mi_attn_fwd_args*>(args), stream);
-      case 1: return mi_attn_fwd_blocksparse(static_cast<const mi_attn_sparse_args*>(args), stream);
-      case 2: return mi_decode(static_cast<const mi_decode_args*>(args), stream);
-      case 3: return mi_decode_splitkv(static_cast<const mi_decode_args*>(args), stream);
-      case 5: return mi_attn_bwd(static_cast<const mi_attn_bwd_args*>(args), stream);
-      case 6: return mi_rmsnorm_fwd(static_cast<const mi_rmsnorm_args*>(args), stream);
-      case 7: return mi_rmsnorm_bwd(static_cast<const mi_rmsnorm_args*>(args), stream);
-      case 8: return mi_xent_fwd(static_cast<const mi_xent_args*>(args), stream);
-      case 9: return mi_xent_dlogits(static_cast<const mi_xent_grad_args*>(args), stream);
-      case 10: return mi_xent_bwd_dlogits(static_cast<const mi_xent_bwd_args*>(args), stream);
-      default: return mi_decode_merge(static_cast<const mi_decode_args*>(args), stream);
-    }
-  };
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  for (int i = 0; i < warmup; ++i) {
-    int rc = once();
-    if (rc) return rc;
-  }
-  hipEvent_t e0, e1;
-  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)
-    return fail(MI_ERR_NO_DEVICE, "hipEventCreate failed");
-  int rc = MI_OK;
-  (void)hipEventRecord(e0, s);
-  for (int i = 0; i < iters && rc == MI_OK; ++i) rc = once();
-  (void)hipEventRecord(e1, s);
-  hipError_t e = hipEventSynchronize(e1);
-  float ms = 0.f;
-  if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-  (void)hipEventDestroy(e0);
-  (void)hipEventDestroy(e1);
-  if (rc) return rc;
-  if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "timing failed: %s", hipGetErrorString(e));
-  *ms_per_launch = ms / iters;
-  return MI_OK;
-}
+int mi_device_cu_count(void) { return mi::device_cu_count(); }
 
 }  // extern "C"

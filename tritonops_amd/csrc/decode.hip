@@ -349,26 +349,14 @@ decode_merge_kernel(const DecodeParams p, int D) {
   if (d == 0 && p.lse) p.lse[(int64_t)b * p.hq + h] = den > 0.f ? M + fast_log2(den) : -INFINITY;
 }
 
-// CUs of the current device (cached per device; 256 if the query fails)
-int decode_cu_count() {
-  static int cached[64] = {0};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached[dev] = n;
-  }
-  return cached[dev];
-}
-
 template <typename T, int D>
 int launch_split(const DecodeParams& p, hipStream_t s) {
   dim3 grid(p.n_splits, p.hkv, p.batch);
   if (p.block_idx == nullptr) {
     // dense: one resident round (8 wavefronts per CU), fewer when there are fewer chunks
     const long long slots = (long long)p.n_splits * p.hkv * p.batch;
-    const long long resident = 8LL * decode_cu_count();
+    const int cus = device_cu_count();
+    const long long resident = 8LL * (cus > 0 ? cus : 256);
     grid = dim3((unsigned)(slots < resident ? slots : resident), 1, 1);
   }
   hipLaunchKernelGGL((decode_splitkv_kernel<T, D>), grid, dim3(64), 0, s, p);

@@ -28,6 +28,23 @@ def window_block_mask(n_blocks, local_window, global_window):
     return causal & (sink | local)
 
 
+_WINDOW_CSR = {}
+
+
+def window_csr(n_blocks, local_window, global_window, device):
+    """CSR (row_ptr, col_idx, strides) of window_block_mask on `device`, built
+    once per (n_blocks, windows, device) and kept: a layer calls with the same
+    windows every step, so nothing is rebuilt or copied to the device per call."""
+    key = (int(n_blocks), int(local_window), int(global_window), str(torch.device(device)))
+    hit = _WINDOW_CSR.get(key)
+    if hit is None:
+        if len(_WINDOW_CSR) >= 64:
+            _WINDOW_CSR.clear()
+        hit = block_mask_to_csr(window_block_mask(*key[:3]), device)
+        _WINDOW_CSR[key] = hit
+    return hit
+
+
 def block_mask_to_csr(mask, device):
     """mask: bool array/tensor [..., nq, nk] with up to two leading (batch,
     head) axes.  Returns (row_ptr, col_idx, strides) where strides =
@@ -48,11 +65,11 @@ def block_mask_to_csr(mask, device):
     row_ptr = np.zeros((B, H, nq + 1), dtype=np.int32)
     row_ptr[..., 1:] = np.cumsum(counts, -1)
     cap = max(int(row_ptr[..., -1].max()), 1)
-    col_idx = np.zeros((B, H, cap), dtype=np.int32)
-    for b in range(B):
-        for h in range(H):
-            cols = np.nonzero(m[b, h])[1]                # row-major => ascending per row
-            col_idx[b, h, : cols.size] = cols
+    col_idx = np.zeros((B * H, cap), dtype=np.int32)
+    unit, _, cols = np.nonzero(m.reshape(B * H, nq, nq))  # row-major => ascending per row
+    first = np.concatenate(([0], np.cumsum(row_ptr[..., -1].reshape(-1))[:-1]))
+    col_idx[unit, np.arange(unit.size) - first[unit]] = cols
+    col_idx = col_idx.reshape(B, H, cap)
     strides = (
         0 if B == 1 else H * (nq + 1), 0 if H == 1 else (nq + 1),
         0 if B == 1 else H * cap, 0 if H == 1 else cap,

@@ -14,7 +14,17 @@ from . import _lib
 from . import masks as _masks
 
 LOG2E = 1.4426950408889634
-_NUM_CUS = 256
+_CU_COUNT = {}
+
+
+def _num_cus(lib):
+    """Compute units of the current device, as the library's own launches see
+    them (cached per device)."""
+    dev = torch.cuda.current_device()
+    n = _CU_COUNT.get(dev)
+    if n is None:
+        n = _CU_COUNT[dev] = int(lib.mi_device_cu_count())
+    return n
 
 
 def _dtype_tag(t):
@@ -69,6 +79,23 @@ def _pad_last(t, Dp):
     return t if t.shape[-1] == Dp else torch.nn.functional.pad(t, (0, Dp - t.shape[-1]))
 
 
+def _check_qkv(q, k, v):
+    """Extents of k and v against q, all as [X, S, H, D]: the kernels take every
+    extent from q, so a shorter k or v would be read past its end."""
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("q, k and v must be 4-dimensional")
+    if k.shape[-1] != q.shape[-1] or v.shape[-1] != q.shape[-1]:
+        raise ValueError("q, k and v must share head_dim (got %d, %d, %d)" % (q.shape[-1], k.shape[-1], v.shape[-1]))
+    if k.shape[:2] != q.shape[:2]:
+        raise ValueError("k %s must have the batch and sequence extents of q %s" % (tuple(k.shape), tuple(q.shape)))
+    if v.shape != k.shape:
+        raise ValueError("v %s must have the shape of k %s" % (tuple(v.shape), tuple(k.shape)))
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError("q, k and v must share one dtype (got %s, %s, %s)" % (q.dtype, k.dtype, v.dtype))
+    if k.shape[2] == 0 or q.shape[2] % max(k.shape[2], 1) != 0:
+        raise ValueError("heads_q %d must be a positive multiple of heads_kv %d" % (q.shape[2], k.shape[2]))
+
+
 def _fill_qkvo(a, q, k, v, o, lse, packed):
     """q/k/v/o given as [X, S, H, D] views (X = 1 packed, X = B batched)."""
     a.q, a.k, a.v, a.o, a.lse = _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse)
@@ -86,13 +113,12 @@ def _dense_fwd(q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, want_lse=T
     """q,k,v as [X, S, H, D] (see _fill_qkvo). Returns (o, lse[X, S, H]); with
     `bhsd` the outputs own [X, H, S, D] / [X, H, S] memory and are returned as
     [X, S, H, ...] views of it."""
+    _check_qkv(q, k, v)
     _require_gpu(q, k, v, cu_seq_lens)
     lib = _lib.load()
     q, k, v = _inner_contig(q), _inner_contig(k), _inner_contig(v)
     packed = cu_seq_lens is not None
     X, S, Hq, D = q.shape
-    if k.shape[-1] != D or v.shape[-1] != D:
-        raise ValueError("q, k and v must share head_dim (got %d, %d, %d)" % (D, k.shape[-1], v.shape[-1]))
     Dp = _padded_head_dim(D)
     if Dp != D:
         o, lse = _dense_fwd(_pad_last(q, Dp), _pad_last(k, Dp), _pad_last(v, Dp), cu_seq_lens, scale_log2, causal,
@@ -103,6 +129,12 @@ def _dense_fwd(q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, want_lse=T
     if bhsd:
         o = torch.empty((X, Hq, S, D), device=q.device, dtype=q.dtype).transpose(1, 2)
         lse = torch.empty((X, Hq, S), device=q.device, dtype=torch.float32).transpose(1, 2) if want_lse else None
+    elif packed:
+        # rows outside every sequence (padding behind cu_seq_lens[-1]) are never
+        # written by the kernel: the reference zero-fills both outputs
+        # (flash_attn_triton.py:608-609)
+        o = torch.zeros((X, S, Hq, D), device=q.device, dtype=q.dtype)
+        lse = torch.zeros((X, S, Hq), device=q.device, dtype=torch.float32) if want_lse else None
     else:
         o = torch.empty((X, S, Hq, D), device=q.device, dtype=q.dtype)
         lse = torch.empty((X, S, Hq), device=q.device, dtype=torch.float32) if want_lse else None
@@ -130,9 +162,17 @@ def _dense_fwd(q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, want_lse=T
     return o, lse
 
 
-def _dense_bwd(q, k, v, o, lse, do, cu_seq_lens, scale_log2, causal, max_seq_len):
+def _dense_bwd(q, k, v, o, do, lse, cu_seq_lens, scale_log2, causal, max_seq_len):
     """q, k, v, o, do as [X, S, H, D] views, lse [X, S, H] (see _fill_qkvo).
     Returns dq, dk, dv shaped and laid out like q, k, v."""
+    _check_qkv(q, k, v)
+    if o.shape != q.shape or do.shape != q.shape:
+        raise ValueError("o %s and do %s must have the shape of q %s" % (tuple(o.shape), tuple(do.shape), tuple(q.shape)))
+    if o.dtype != q.dtype or do.dtype != q.dtype:
+        raise ValueError("o and do must have the dtype of q (%s), got %s and %s" % (q.dtype, o.dtype, do.dtype))
+    if lse.shape != q.shape[:3] or lse.dtype != torch.float32:
+        raise ValueError("lse must be float32 %s as returned by the forward, got %s %s"
+                         % (tuple(q.shape[:3]), lse.dtype, tuple(lse.shape)))
     _require_gpu(q, k, v, o, do, lse, cu_seq_lens)
     lib = _lib.load()
     q, k, v, o, do = (_inner_contig(t) for t in (q, k, v, o, do))
@@ -140,7 +180,7 @@ def _dense_bwd(q, k, v, o, lse, do, cu_seq_lens, scale_log2, causal, max_seq_len
     X, S, Hq, D = q.shape
     Dp = _padded_head_dim(D)
     if Dp != D:
-        grads = _dense_bwd(*(_pad_last(t, Dp) for t in (q, k, v, o)), lse, _pad_last(do, Dp), cu_seq_lens,
+        grads = _dense_bwd(*(_pad_last(t, Dp) for t in (q, k, v, o, do)), lse, cu_seq_lens,
                            scale_log2, causal, max_seq_len)
         return tuple(g[..., :D].contiguous() for g in grads)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
@@ -176,12 +216,13 @@ def _dense_bwd(q, k, v, o, lse, do, cu_seq_lens, scale_log2, causal, max_seq_len
     return dq, dk, dv
 
 
-def flash_attn_triton_bwd(q, k, v, o, lse, do, cu_seq_lens, sm_scale, *, max_seq_len=None):
-    """Causal var-len GQA backward on packed tensors: contract of
-    flash_attn_triton_bwd in flash_attn_triton/flash_attn_triton.py:661-813
-    (`sm_scale` contains log2(e), `lse` is the base-2 LSE the forward returned).
-    Returns (dq, dk, dv) with the shapes of q, k, v."""
-    return _dense_bwd(q, k, v, o, lse, do, cu_seq_lens, sm_scale, True, max_seq_len)
+def flash_attn_triton_bwd(q, k, v, o, do, lse, cu_seq_lens, sm_scale, *, max_seq_len=None):
+    """Causal var-len GQA backward on packed tensors: contract and argument
+    order of flash_attn_triton_bwd in flash_attn_triton/flash_attn_triton.py
+    :661-670 (`do` before `lse`; `sm_scale` contains log2(e), `lse` is the
+    base-2 LSE the forward returned).  Returns (dq, dk, dv) with the shapes of
+    q, k, v; rows outside every sequence receive zeros."""
+    return _dense_bwd(q, k, v, o, do, lse, cu_seq_lens, sm_scale, True, max_seq_len)
 
 
 def flash_attn_triton_fwd(q, k, v, cu_seq_lens, sm_scale, *, max_seq_len=None):
@@ -191,8 +232,10 @@ def flash_attn_triton_fwd(q, k, v, cu_seq_lens, sm_scale, *, max_seq_len=None):
     flash_attn_triton/flash_attn_triton.py:595-658: q [1,T,Hq,D], k/v
     [1,T,Hkv,D], cu_seq_lens [B+1]; `sm_scale` already contains log2(e)
     (:839).  Returns (o [1,T,Hq,D], lse [1,T,Hq] fp32, base 2).  Rows outside
-    every sequence are left unwritten (the reference zero-fills them).
-    `max_seq_len` skips the host sync that sizes the grid (:621).
+    every sequence are zero in both, as in the reference (:608-609).
+    `max_seq_len` skips the host sync that sizes the grid (:621); it must be
+    an upper bound of every sequence length (rows beyond it may or may not be
+    computed).
     """
     return _dense_fwd(q, k, v, cu_seq_lens, sm_scale, True, max_seq_len)
 
@@ -213,7 +256,7 @@ class flash_attn_triton(torch.autograd.Function):
     @staticmethod
     def backward(ctx, do):
         q, k, v, o, lse, cu_seq_lens = ctx.saved_tensors
-        dq, dk, dv = flash_attn_triton_bwd(q, k, v, o, lse, do, cu_seq_lens, ctx.sm_scale)
+        dq, dk, dv = flash_attn_triton_bwd(q, k, v, o, do, lse, cu_seq_lens, ctx.sm_scale)
         return dq, dk, dv, None
 
 
@@ -234,7 +277,7 @@ class _FlashAttention(torch.autograd.Function):
     def backward(ctx, do, _dlse):
         q, k, v, o, lse, cu_seq_lens = ctx.saved_tensors
         scale_log2, causal, max_seq_len = ctx.opts
-        dq, dk, dv = _dense_bwd(q, k, v, o, lse, do, cu_seq_lens, scale_log2, causal, max_seq_len)
+        dq, dk, dv = _dense_bwd(q, k, v, o, do, lse, cu_seq_lens, scale_log2, causal, max_seq_len)
         return dq, dk, dv, None, None, None, None, None
 
 
@@ -293,6 +336,10 @@ def flash_attn_sparse_triton(q, k, v, cu_seqlens, softmax_scale=None, local_wind
     `csr_strides`); diagonal blocks are masked causally per token.
     A query with no allowed key gets o = 0 and lse = -inf.
     """
+    if cu_seqlens is not None:
+        _check_qkv(q, k, v)
+    else:
+        _check_qkv(*(t.transpose(1, 2) if t.dim() == 4 else t for t in (q, k, v)))
     _require_gpu(q, k, v, cu_seqlens)
     lib = _lib.load()
     D0 = q.shape[-1]
@@ -311,8 +358,10 @@ def flash_attn_sparse_triton(q, k, v, cu_seqlens, softmax_scale=None, local_wind
             raise ValueError("packed layout expects a leading dimension of 1")
         cu = cu_seqlens.to(torch.int32)
         max_len = min(_max_len(cu, max_seq_len), T)
-        o = torch.empty_like(q)
-        lse = torch.empty((1, T, Hq), device=q.device, dtype=torch.float32)
+        # rows outside every sequence are not written by the kernel; zero like the
+        # reference (flash_attn_sparse_attn_triton.py:274-275)
+        o = torch.zeros_like(q)
+        lse = torch.zeros((1, T, Hq), device=q.device, dtype=torch.float32)
         qv, kv, vv, ov, lv = q, k, v, o, lse
         batch = cu.numel() - 1
     else:
@@ -332,8 +381,9 @@ def flash_attn_sparse_triton(q, k, v, cu_seqlens, softmax_scale=None, local_wind
             wl, wg = int(local_window_size), int(global_window_size)
             if wl < 0 or wg < 0:
                 raise ValueError("window sizes must be >= 0")
-            block_mask = _masks.window_block_mask(nqb, wl, wg)
-        row_ptr, col_idx, csr_strides = _masks.block_mask_to_csr(block_mask, q.device)
+            row_ptr, col_idx, csr_strides = _masks.window_csr(nqb, wl, wg, q.device)
+        else:
+            row_ptr, col_idx, csr_strides = _masks.block_mask_to_csr(block_mask, q.device)
         if row_ptr.shape[-1] - 1 < nqb:
             raise ValueError("block mask covers %d query blocks, sequences need %d" % (row_ptr.shape[-1] - 1, nqb))
     if q.numel() == 0:
@@ -358,10 +408,23 @@ def flash_attn_sparse_triton(q, k, v, cu_seqlens, softmax_scale=None, local_wind
 def _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, return_lse,
             block_idx=None, block_cnt=None, bi_strides=(0, 0), max_blocks=0, split_blocks=0,
             window=(-1, -1), include_last=False, kv_layout="batched", page_table=None, page_size=0):
-    _require_gpu(q, k, v, cu_seq_lens, seq_lens, page_table)
-    lib = _lib.load()
-    if v.shape[-1] != q.shape[-1] or k.shape[-1] != q.shape[-1]:
+    if q.dim() != 3 or k.dim() != 4:
+        raise ValueError("decoding takes q [B, Hq, D] and k, v [B, maxL, Hkv, D] (or a packed / paged cache)")
+    if v.shape != k.shape:
+        raise ValueError("v %s must have the shape of k %s" % (tuple(v.shape), tuple(k.shape)))
+    if k.shape[-1] != q.shape[-1]:
         raise ValueError("q, k and v must share head_dim")
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError("q, k and v must share one dtype (got %s, %s, %s)" % (q.dtype, k.dtype, v.dtype))
+    if k.shape[2] == 0 or q.shape[1] % k.shape[2] != 0:
+        raise ValueError("heads_q %d must be a positive multiple of heads_kv %d" % (q.shape[1], k.shape[2]))
+    for name, t, n in (("cu_seq_lens", cu_seq_lens, q.shape[0] + 1), ("seq_lens", seq_lens, q.shape[0])):
+        if t is not None and (t.dim() != 1 or t.numel() != n or t.is_floating_point()):
+            raise ValueError("%s must be an integer tensor of %d entries" % (name, n))
+    if page_table is not None and page_table.is_floating_point():
+        raise ValueError("page_table must be an integer tensor")
+    _require_gpu(q, k, v, cu_seq_lens, seq_lens, page_table, block_idx, block_cnt)
+    lib = _lib.load()
     D0 = q.shape[-1]
     if _padded_head_dim(D0) != D0:
         # zero-padded copies of the cache: correct, but a cache that is decoded from
@@ -429,7 +492,7 @@ def _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, re
     a.scale_log2 = float(scale) * LOG2E
     if block_idx is None:
         a.split_tokens = int(split_tokens) if split_tokens else lib.mi_decode_choose_split_tokens(
-            B, Hkv, a.max_seqlen, _NUM_CUS)
+            B, Hkv, a.max_seqlen, _num_cus(lib))
     else:
         a.split_tokens = 64
         a.block_idx, a.block_cnt = _ptr(block_idx), _ptr(block_cnt)
@@ -438,7 +501,7 @@ def _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, re
         a.include_last_block = 1 if include_last else 0
         a.max_blocks, a.block_size = int(max_blocks), _masks.BLOCK
         a.split_blocks = int(split_blocks) if split_blocks else lib.mi_decode_choose_split_blocks(
-            B, Hkv, a.max_blocks + a.include_last_block, _NUM_CUS)
+            B, Hkv, a.max_blocks + a.include_last_block, _num_cus(lib))
     nbytes = lib.mi_decode_workspace_bytes(C.byref(a))
     if nbytes == 0:
         raise _lib.MiAttnError(lib.mi_decode_validate(C.byref(a)), lib.mi_last_error().decode())
@@ -527,11 +590,24 @@ def flash_attention_sparse_decoding(q, k, v, cu_seq_lens, global_window_size=64,
         return _decode(q, k, v, None, lens, scale, None, None, return_lse, block_idx=idx, block_cnt=cnt,
                        bi_strides=(cap, 0), max_blocks=cap,
                        split_blocks=split_blocks or 0, window=(lw, gw), **layout)
+    if block_indices.dim() != 3 or block_indices.shape[0] != B or block_indices.shape[1] != Hkv \
+            or block_indices.is_floating_point():
+        raise ValueError("block_indices must be an integer tensor [B, Hkv, n], got %s %s"
+                         % (block_indices.dtype, tuple(block_indices.shape)))
     idx = block_indices.to(torch.int32).contiguous()
-    if idx.dim() != 3 or idx.shape[0] != B or idx.shape[1] != Hkv:
-        raise ValueError("block_indices must be [B, Hkv, n]")
     n = idx.shape[2]
-    cnt = block_counts.to(torch.int32).contiguous() if block_counts is not None else None
+    cnt = None
+    if block_counts is not None:
+        if block_counts.shape != (B, Hkv) or block_counts.is_floating_point():
+            raise ValueError("block_counts must be an integer tensor [B, Hkv]")
+        cnt = block_counts.to(torch.int32).contiguous()
+    if n == 0:
+        if not include_last_block:
+            raise ValueError("an empty block list needs include_last_block")
+        # a non-NULL list address selects the block form even when only the implicit block is read
+        idx = torch.zeros((B, Hkv, 1), device=q.device, dtype=torch.int32)
+        return _decode(q, k, v, None, lens, scale, None, None, return_lse, block_idx=idx, block_cnt=None,
+                       bi_strides=(Hkv, 1), max_blocks=0, split_blocks=split_blocks or 0, include_last=True, **layout)
     # the block of the newest token is appended (and de-duplicated) by the kernel
     return _decode(q, k, v, None, lens, scale, None, None, return_lse, block_idx=idx, block_cnt=cnt,
                    bi_strides=(Hkv * n, n), max_blocks=n, split_blocks=split_blocks or 0,
