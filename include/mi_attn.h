@@ -296,6 +296,25 @@ int mi_decode_merge(const mi_decode_args *args, void *stream);
 /* Both passes back to back on `stream`. */
 int mi_decode(const mi_decode_args *args, void *stream);
 
+/* mi_decode for callers that cannot allocate device memory.
+ * No counterpart in the reference (its launcher allocates the partial results
+ * with torch on every call, flash_attn_decoding.py:249-261).  It is for callers
+ * that cannot call hipMalloc or size and carry a workspace: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid allocation.
+ * Same arguments and results (bit for bit) as mi_decode, except that
+ * args->workspace / workspace_bytes are ignored: the split-KV partials go to a
+ * buffer of MI_DECODE_STATIC_SCRATCH_BYTES that the library holds in device
+ * memory, one per GPU, from load time until the process ends.  A call whose
+ * mi_decode_workspace_bytes() exceeds that size fails with MI_ERR_WORKSPACE
+ * before anything is launched (pick larger split_tokens / split_blocks).
+ * The call allocates and frees nothing and records only kernel launches.
+ * Every call on one GPU uses the same buffer: calls that overlap on one GPU
+ * (different streams, or graphs replayed concurrently) race; serialise them.
+ * The buffer keeps the previous call's partials; nothing in it needs to start
+ * at zero, because pass 2 reads only the slots pass 1 of the same call wrote. */
+#define MI_DECODE_STATIC_SCRATCH_BYTES (32u << 20)
+int mi_decode_noalloc(const mi_decode_args *args, void *stream);
+
 /* ------------------------------------------------------------------------- */
 /* RMSNorm forward / backward over rows of `dim` elements.
  * Replaces RMSNormTritonFunction.forward / .backward and their kernels

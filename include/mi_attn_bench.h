@@ -21,7 +21,7 @@ extern "C" {
  * kind: 0 = mi_attn_fwd, 1 = mi_attn_fwd_blocksparse, 2 = mi_decode,
  *       3 = mi_decode_splitkv, 4 = mi_decode_merge, 5 = mi_attn_bwd,
  *       6 = mi_rmsnorm_fwd, 7 = mi_rmsnorm_bwd, 8 = mi_xent_fwd,
- *       9 = mi_xent_dlogits, 10 = mi_xent_bwd_dlogits.
+ *       9 = mi_xent_dlogits, 10 = mi_xent_bwd_dlogits, 11 = mi_decode_noalloc.
  * `args` points to `n_args` argument structs of that entry point laid out
  * `arg_stride` bytes apart; launch i uses struct i % n_args, so a benchmark can
  * rotate inputs that would otherwise stay in the last-level cache.

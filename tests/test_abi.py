@@ -200,6 +200,23 @@ def test_decode_geometry_and_validation(lib):
     assert lib.mi_status_name(lib.mi_decode_validate(C.byref(a))).decode() == "MI_ERR_SPARSE_LAYOUT"
 
 
+def test_decode_noalloc_validation(lib):
+    """The entry point that allocates nothing ignores the workspace fields and
+    refuses, before any HIP call, a launch whose partials exceed its buffer."""
+    a = _good_decode()
+    a.workspace, a.workspace_bytes = None, 0
+    a.head_dim = 32                                   # every other check still runs first
+    assert lib.mi_status_name(lib.mi_decode_noalloc(C.byref(a), None)).decode() == "MI_ERR_HEAD_DIM"
+    a = _good_decode()
+    a.workspace, a.workspace_bytes = None, 0
+    a.batch, a.max_seqlen, a.split_tokens = 64, 1 << 20, 64      # 64 * 32 * 16384 * 129 * 4 bytes of partials
+    assert lib.mi_decode_workspace_bytes(C.byref(a)) > _lib.MI_DECODE_STATIC_SCRATCH_BYTES
+    rc = lib.mi_decode_noalloc(C.byref(a), None)
+    assert lib.mi_status_name(rc).decode() == "MI_ERR_WORKSPACE" and "static buffer" in _err(lib)
+    text = open(HEADERS[0]).read()
+    assert re.search(r"#define MI_DECODE_STATIC_SCRATCH_BYTES \(32u << 20\)", text)
+
+
 def test_decode_kv_layout_validation(lib):
     a = _good_decode()
     a.kv_layout = 7

@@ -10,6 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmi_attn.so")
 
 MI_ATTN_ABI_VERSION = 5
+MI_DECODE_STATIC_SCRATCH_BYTES = 32 << 20
 MI_KV_BATCHED, MI_KV_PACKED, MI_KV_PAGED = 0, 1, 2
 MI_ATTN_BLOCK = 64
 MI_DTYPE_F32 = 2
@@ -178,6 +179,7 @@ EXPORTS = {
     "mi_attn_fwd_validate": (C.c_int, [C.POINTER(AttnFwdArgs)]),
     "mi_attn_fwd_blocksparse_validate": (C.c_int, [C.POINTER(AttnSparseArgs)]),
     "mi_decode_validate": (C.c_int, [C.POINTER(DecodeArgs)]),
+    "mi_decode_noalloc": (C.c_int, [C.POINTER(DecodeArgs), _vp]),
     "mi_device_cu_count": (C.c_int, []),
     # include/mi_attn_bench.h
     "mi_time_launches": (C.c_int, [C.c_int, _vp, C.c_int, _sz, _vp, C.c_int, C.c_int, C.POINTER(C.c_float)]),

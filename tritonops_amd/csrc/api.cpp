@@ -431,6 +431,8 @@ int mi_attn_fwd_blocksparse(const mi_attn_sparse_args* a, void* stream) {
   return launch_status(mi::launch_prefill_sparse(p, a->dtype, a->head_dim, static_cast<hipStream_t>(stream)), "mi_attn_fwd_blocksparse");
 }
 
+static_assert(mi::kDecodeScratchBytes == MI_DECODE_STATIC_SCRATCH_BYTES, "header and kernel disagree on the static buffer");
+
 static int decode_validate_shape(const mi_decode_args* a) {
   if (!a) return fail(MI_ERR_NULL_POINTER, "args is NULL");
   if (a->struct_size != sizeof(mi_decode_args))
@@ -562,6 +564,25 @@ int mi_decode(const mi_decode_args* a, void* stream) {
   int rc = mi_decode_splitkv(a, stream);
   if (rc) return rc;
   return mi_decode_merge(a, stream);
+}
+
+int mi_decode_noalloc(const mi_decode_args* a, void* stream) {
+  int rc = decode_validate_args(a);
+  if (rc) return rc;
+  const size_t need = mi_decode_workspace_bytes(a);
+  if (need > MI_DECODE_STATIC_SCRATCH_BYTES)
+    return fail(MI_ERR_WORKSPACE,
+                "the split-KV partials of this call take %zu bytes, the static buffer of mi_decode_noalloc holds %u: "
+                "use larger split_tokens / split_blocks or mi_decode with a workspace",
+                need, (unsigned)MI_DECODE_STATIC_SCRATCH_BYTES);
+  void* buf = nullptr;
+  const int e = mi::decode_static_scratch(&buf);
+  if (e != 0) return fail(MI_ERR_NO_DEVICE, "device address of the static decode buffer: %s",
+                          hipGetErrorString(static_cast<hipError_t>(e)));
+  mi_decode_args b = *a;
+  b.workspace = buf;
+  b.workspace_bytes = MI_DECODE_STATIC_SCRATCH_BYTES;
+  return mi_decode(&b, stream);
 }
 
 int mi_device_cu_count(void) { return mi::device_cu_count(); }

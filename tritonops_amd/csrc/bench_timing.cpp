@@ -6,7 +6,7 @@
 
 extern "C" int mi_time_launches(int kind, const void* args, int n_args, size_t arg_stride, void* stream, int warmup,
                                 int iters, float* ms_per_launch) {
-  if (!args || !ms_per_launch || n_args <= 0 || iters <= 0 || warmup < 0 || kind < 0 || kind > 10)
+  if (!args || !ms_per_launch || n_args <= 0 || iters <= 0 || warmup < 0 || kind < 0 || kind > 11)
     return MI_ERR_SHAPE;
   const char* base = static_cast<const char*>(args);
   int n = 0;
@@ -23,7 +23,8 @@ extern "C" int mi_time_launches(int kind, const void* args, int n_args, size_t a
       case 7: return mi_rmsnorm_bwd(static_cast<const mi_rmsnorm_args*>(a), stream);
       case 8: return mi_xent_fwd(static_cast<const mi_xent_args*>(a), stream);
       case 9: return mi_xent_dlogits(static_cast<const mi_xent_grad_args*>(a), stream);
-      default: return mi_xent_bwd_dlogits(static_cast<const mi_xent_bwd_args*>(a), stream);
+      case 10: return mi_xent_bwd_dlogits(static_cast<const mi_xent_bwd_args*>(a), stream);
+      default: return mi_decode_noalloc(static_cast<const mi_decode_args*>(a), stream);
     }
   };
   hipStream_t s = static_cast<hipStream_t>(stream);

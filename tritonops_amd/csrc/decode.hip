@@ -21,8 +21,16 @@
 // single wave's LDS operations execute in order.  Partials are fp32 (the reference
 // rounds them to the input dtype, :249-251).
 // Pass 2: per (sequence, q-head) merge  o = sum_c o_c 2^(lse_c - lse).
+#include <atomic>
+
 #include "kernels.h"
 #include "tile_core.h"
+
+// Split-KV partials of mi_decode_noalloc: device memory the library holds from
+// load time on, one copy per GPU.  Host code must not use this name as an
+// address (it is a host-side stand-in); decode_static_scratch() below asks the
+// runtime for the device address, per device, and everything else uses that.
+static __device__ __align__(256) unsigned char scratch[mi::kDecodeScratchBytes];
 
 namespace mi {
 namespace {
@@ -364,6 +372,28 @@ int launch_split(const DecodeParams& p, hipStream_t s) {
 }
 
 }  // namespace
+
+// Device address of `scratch` on the current device.  Looked up once per device
+// with that device current (each GPU holds its own copy at its own address);
+// the lookup allocates nothing.  Two threads racing on the first call both
+// look it up and store the same value.
+int decode_static_scratch(void** ptr) {
+  constexpr int kMaxDev = 64;
+  static std::atomic<void*> addr[kMaxDev];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDev) return (int)hipErrorInvalidDevice;
+  void* a = addr[dev].load(std::memory_order_acquire);
+  if (a == nullptr) {
+    e = hipGetSymbolAddress(&a, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (a == nullptr) return (int)hipErrorInvalidSymbol;
+    addr[dev].store(a, std::memory_order_release);
+  }
+  *ptr = a;
+  return (int)hipSuccess;
+}
 
 int launch_decode_splitkv(const DecodeParams& p, int dtype, int head_dim, hipStream_t s) {
   if (dtype == 0) {

@@ -128,6 +128,11 @@ int launch_prefill_dense(const PrefillParams& p, int dtype, int head_dim, hipStr
 int launch_prefill_sparse(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);
 int launch_decode_splitkv(const DecodeParams& p, int dtype, int head_dim, hipStream_t s);
 int launch_decode_merge(const DecodeParams& p, int dtype, int head_dim, hipStream_t s);
+// Bytes of the static device buffer behind mi_decode_noalloc
+// (= MI_DECODE_STATIC_SCRATCH_BYTES) and its device address on the current
+// device (hipError_t as int; no allocation).
+constexpr unsigned kDecodeScratchBytes = 32u << 20;
+int decode_static_scratch(void** ptr);
 // delta, dq, dk, dv kernels in that order
 int launch_attn_bwd(const BwdParams& p, int dtype, int head_dim, hipStream_t s);
 // RMSNorm.  x_dtype: 0 bf16, 1 f16, 2 f32; w_dtype: x_dtype or 2.  `vec`: rows
