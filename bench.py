@@ -13,8 +13,10 @@ A step is one pass of the path over one batch of synthetic inputs that are
 already resident in HBM.  `value` comes from wall-clock around K steps
 bracketed by device synchronisation; `roofline.achieved` comes from HIP events
 recorded on the launch stream around the same kernels (mi_time_launches).
-The CPU baseline is the reference's PyTorch attention math (oracle/) timed on
-this host's cores on a stated slice of the same workload.
+`max_abs_err` is the largest |kernel - fp32 torch math| over a stated sample of
+the benchmark tensors themselves (rows / heads / sequences), computed on the
+device.  The CPU baseline is the reference's PyTorch attention math (oracle/)
+timed on this host's cores on a stated slice of the same workload.
 """
 import argparse
 import ctypes as C
@@ -31,6 +33,25 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+# Device symbols of the kernels each workload's roofline figure is about, as
+# rocprofv3 prints them (it leaves names with a bf16 template argument mangled).
+# tests/test_abi.py checks that the built library contains every one of them.
+_NS = "_ZN2mi12_GLOBAL__N_1"
+KERNELS = {
+    "dense_causal": _NS + "12dense_kernelIDF16bLi128EEEvNS_13PrefillParamsE",
+    "c1_dense_noncausal_small": _NS + "12dense_kernelIDF16bLi64EEEvNS_13PrefillParamsE",
+    "gqa_decode": _NS + "21decode_splitkv_kernelIDF16bLi128EEEvNS_12DecodeParamsE",
+    "block_sparse": _NS + "13sparse_kernelIDF16bLi128ELi2ELi2ELi32EEEvNS_13PrefillParamsE",
+    "sparse_decode": _NS + "21decode_splitkv_kernelIDF16bLi128EEEvNS_12DecodeParamsE",
+    "dense_causal_bwd": " + ".join(_NS + n for n in (
+        "16bwd_delta_kernelIDF16bEEvNS_9BwdParamsEi", "10bwd_kernelIDF16bLi128ELi0EEEvNS_9BwdParamsEi",
+        "10bwd_kernelIDF16bLi128ELi1EEEvNS_9BwdParamsEi", "10bwd_kernelIDF16bLi128ELi2EEEvNS_9BwdParamsEi")),
+    "rmsnorm": " + ".join(_NS + n for n in (
+        "18rms_fwd_vec_kernelIDF16bfLi2ELi4EEEvNS_9RmsParamsE", "18rms_bwd_vec_kernelIDF16bfLi2ELi4EEEvNS_9RmsParamsE",
+        "19rms_dw_stage_kernelILi4EEEvPKfPfii", "20rms_dw_reduce_kernelIfEEvPKfPT_ii")),
+    "fused_xent": _NS + "16xent_gemm_kernelIDF16bLb0EEEvNS_10XentParamsE",
+}
 
 
 def _sync():
@@ -76,6 +97,21 @@ def _event_ms(kind, args, steps, warmup):
     return ms.value
 
 
+def _ref_rows(q, k, v, rows, scale, allow):
+    """fp32 softmax(q k^T scale) v and base-2 LSE on the device: q [..., S, D]
+    restricted to `rows`, k / v [..., S, D], allow bool [len(rows), S]."""
+    s = torch.einsum("...id,...jd->...ij", q[..., rows, :].float(), k.float()) * scale
+    s = s.masked_fill(~allow, float("-inf"))
+    return torch.einsum("...ij,...jd->...id", torch.softmax(s, -1), v.float()), torch.logsumexp(s, -1) * LOG2E
+
+
+def _err(got, want):
+    return float((got.float() - want.float()).abs().max().item())
+
+
+LOG2E = 1.4426950408889634
+
+
 # ----------------------------------------------------------------------------
 # workloads: each returns dict(ms_per_step, kernel_ms, work, unit-specific...)
 # ----------------------------------------------------------------------------
@@ -109,13 +145,52 @@ def run_dense_causal(steps, warmup):
     lse = torch.empty((B, H, S), device="cuda", dtype=torch.float32)
     kms = _event_ms(0, _fwd_args(q, k, v, o, lse, True), steps, warmup)
     flop = 2.0 * B * H * S * (S + 1) * D            # 4*D per unmasked (q, k) pair
+    # parity on the benchmark tensors: three (batch, head) units x four 64-row blocks
+    err = err_lse = 0.0
+    keys = torch.arange(S, device="cuda")
+    for b, h in ((0, 0), (1, 13), (3, 31)):
+        for r0 in (0, 1984, 4096, S - 64):
+            rows = torch.arange(r0, r0 + 64, device="cuda")
+            want, want_lse = _ref_rows(q[b, h], k[b, h], v[b, h], rows, D ** -0.5, keys[None, :] <= rows[:, None])
+            err = max(err, _err(o[b, h, rows], want))
+            err_lse = max(err_lse, _err(lse[b, h, rows], want_lse))
     return {
         "name": "dense_causal", "ms_per_step": ms, "kernel_ms": kms,
         "metric": "attn_fwd_tflops", "unit": "TFLOP/s", "value": flop / (ms * 1e-3) / 1e12,
+        "max_abs_err": err, "max_abs_err_lse2": err_lse,
+        "err_sample": "o and lse of 3 (batch, head) units x 4 blocks of 64 query rows against fp32 torch math on the device",
         "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "kernel": "dense_kernel<bf16,128>"},
+                     "unit": "TFLOP/s", "kernel": KERNELS["dense_causal"]},
         "config": {"workload": "dense causal flash-attention fwd bf16 B=4 H=32 S=8192 D=128, o bf16 + lse fp32",
                    "flop_per_step": flop, "flop_reference_convention_4BHS2D": 4.0 * B * H * S * S * D},
+    }
+
+
+def run_c1_small(steps, warmup):
+    """The reference's CPU-runnable case: dense non-causal B=1 H=4 S=256 D=64, q/k/v drawn in fp32 on the CPU
+    from seed 0.  The GPU path runs it on the bf16 cast; the parity figure is against fp32 math on the fp32
+    inputs, so it includes the rounding of the inputs."""
+    import tritonops_amd as ta
+    B, H, S, D = 1, 4, 256, 64
+    g = torch.Generator().manual_seed(0)
+    q32, k32, v32 = (torch.randn((B, H, S, D), generator=g) for _ in range(3))
+    q, k, v = (t.to(torch.bfloat16).cuda() for t in (q32, k32, v32))
+    fn = lambda: ta.flash_attention(q, k, v, causal=False, return_lse=True)
+    ms = _time_steps(fn, steps, warmup)
+    o, lse = fn()
+    kms = _event_ms(0, _fwd_args(q, k, v, torch.empty_like(q), torch.empty_like(lse), False), steps, warmup)
+    want = torch.softmax(torch.einsum("bhid,bhjd->bhij", q32, k32) / 8.0, -1) @ v32
+    flop = 4.0 * B * H * S * S * D
+    return {
+        "name": "c1_dense_noncausal_small", "ms_per_step": ms, "kernel_ms": kms,
+        "metric": "attn_fwd_tflops", "unit": "TFLOP/s", "value": flop / (ms * 1e-3) / 1e12,
+        "max_abs_err": _err(o.cpu(), want),
+        "err_sample": "all of o against fp32 softmax(q k^T / 8) v on the fp32 inputs (the kernel sees their bf16 cast)",
+        "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "kernel": KERNELS["c1_dense_noncausal_small"]},
+        "config": {"workload": "dense non-causal attention fwd B=1 H=4 S=256 D=64 (the reference's CPU case; 4 work items, "
+                               "launch-latency bound on a GPU), bf16 cast of fp32 N(0,1) inputs from seed 0",
+                   "flop_per_step": flop},
     }
 
 
@@ -149,11 +224,21 @@ def run_dense_bwd(steps, warmup):
     a.workspace, a.workspace_bytes = ws.data_ptr(), nb
     kms = _event_ms(5, a, steps, warmup)
     flop = 2.5 * 2.0 * B * H * S * (S + 1) * D       # 10*D per unmasked (q, k) pair: S, dP, dV, dQ, dK
+    # parity on the benchmark tensors: one (batch, head) unit through autograd in fp32 on the device
+    b, h = 2, 17
+    qr, kr, vr = (t[b, h].float().requires_grad_(True) for t in (q, k, v))
+    sc = (qr @ kr.T) * D ** -0.5
+    sc = sc.masked_fill(~torch.ones(S, S, dtype=torch.bool, device="cuda").tril(), float("-inf"))
+    (torch.softmax(sc, -1) @ vr).backward(do[b, h].float())
+    err = max(_err(dq[b, :, h], qr.grad), _err(dk[b, :, h], kr.grad), _err(dv[b, :, h], vr.grad))
+    del qr, kr, vr, sc
     return {
         "name": "dense_causal_bwd", "ms_per_step": ms, "kernel_ms": kms,
         "metric": "attn_bwd_tflops", "unit": "TFLOP/s", "value": flop / (ms * 1e-3) / 1e12,
+        "max_abs_err": err,
+        "err_sample": "dq, dk, dv of one (batch, head) unit against autograd through fp32 torch math on the device (bar 3e-2)",
         "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "kernel": "bwd_delta_kernel + bwd_kernel<bf16,128,{dq,dk,dv}> (four launches)"},
+                     "unit": "TFLOP/s", "kernel": KERNELS["dense_causal_bwd"]},
         "config": {"workload": "dense causal attention bwd bf16 B=4 H=32 S=8192 D=128: dq, dk, dv from q, k, v, o, lse, do",
                    "flop_per_step": flop,
                    "note": "the three kernels execute 16*D FLOP per pair (S three times, dP twice); the figure "
@@ -193,12 +278,23 @@ def run_decode(steps, warmup):
     a.seq_lens, a.cu_seqlens = lens_d.data_ptr(), None
     a.batch, a.heads_q, a.heads_kv, a.max_seqlen, a.head_dim = B, Hq, Hkv, L, D
     a.scale_log2 = D ** -0.5 * 1.4426950408889634
-    a.split_tokens = lib.mi_decode_choose_split_tokens(B, Hkv, L, 256)
+    a.split_tokens = lib.mi_decode_choose_split_tokens(B, Hkv, L, lib.mi_device_cu_count())
     nbytes = lib.mi_decode_workspace_bytes(C.byref(a))
     ws = torch.empty(nbytes, device="cuda", dtype=torch.uint8)
     a.workspace, a.workspace_bytes = ws.data_ptr(), nbytes
-    k_split = _event_ms(3, a, steps, warmup)
+    # launches alternate the two caches, like the wall-clock leg
+    a2 = _lib.DecodeArgs.from_buffer_copy(a)
+    a2.k, a2.v = caches[1][0].data_ptr(), caches[1][1].data_ptr()
+    k_split = _event_ms(3, [a, a2], steps, warmup)
     k_merge = _event_ms(4, a, steps, warmup)
+    # parity on the benchmark tensors: three sequences against fp32 torch math on the device
+    got = ta.flash_attention_decoding(q, k, v, None, seq_lens=lens_d)
+    err = 0.0
+    for b in (0, 31, 63):
+        n = int(lens[b])
+        sc = torch.einsum("gid,gld->gil", q[b].view(Hkv, Hq // Hkv, D).float(), kc[b, :, :n].float()) * D ** -0.5
+        want = torch.einsum("gil,gld->gid", torch.softmax(sc, -1), vc[b, :, :n].float()).reshape(Hq, D)
+        err = max(err, _err(got[b], want))
     # same cache as a pool of shuffled 64-token pages [pages, Hkv, 64, D] behind a page table
     ps = 64
     npg = L // ps
@@ -221,8 +317,10 @@ def run_decode(steps, warmup):
     return {
         "name": "gqa_decode", "ms_per_step": ms, "kernel_ms": k_split, "merge_kernel_ms": k_merge,
         "metric": "decode_hbm_gbs", "unit": "GB/s", "value": nbytes_alg / (ms * 1e-3) / 1e9,
+        "max_abs_err": err,
+        "err_sample": "3 of the 64 sequences (all heads) against fp32 torch math on the device",
         "roofline": {"bound": "hbm", "achieved": nbytes_alg / (k_split * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "kernel": "decode_splitkv_kernel<bf16,128>"},
+                     "unit": "GB/s", "kernel": KERNELS["gqa_decode"]},
         "config": {"workload": "GQA decode bf16 B=64 Hq=32 Hkv=8 KV<=32768 (lens U[16384,32768]) D=128, split-KV + LSE merge",
                    "bytes_per_step": nbytes_alg, "split_tokens": int(a.split_tokens),
                    "paged_cache_kernel_ms": k_paged,
@@ -261,11 +359,22 @@ def run_block_sparse(steps, warmup):
     a.scale_log2 = D ** -0.5 * 1.4426950408889634
     kms = _event_ms(1, a, steps, warmup)
     flop = 4.0 * D * ((live - nb) * 64 * 64 + nb * 64 * 65 / 2) * B * H
+    # parity on the benchmark tensors: five query blocks of every (batch, head) unit
+    bm = torch.from_numpy(m).cuda()
+    keys = torch.arange(S, device="cuda")
+    err = err_lse = 0.0
+    for qb in (0, 3, 64, 129, 255):
+        rows = torch.arange(qb * 64, qb * 64 + 64, device="cuda")
+        want, want_lse = _ref_rows(q, k, v, rows, D ** -0.5, bm[qb][keys // 64][None, :] & (keys[None, :] <= rows[:, None]))
+        err = max(err, _err(o[:, :, rows], want))
+        err_lse = max(err_lse, _err(lse[:, :, rows], want_lse))
     return {
         "name": "block_sparse", "ms_per_step": ms, "kernel_ms": kms,
         "metric": "sparse_attn_fwd_tflops", "unit": "TFLOP/s", "value": flop / (ms * 1e-3) / 1e12,
+        "max_abs_err": err, "max_abs_err_lse2": err_lse,
+        "err_sample": "5 of the 256 query blocks of all 32 (batch, head) units against masked fp32 torch math on the device",
         "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "kernel": "sparse_kernel<bf16,128>"},
+                     "unit": "TFLOP/s", "kernel": KERNELS["block_sparse"]},
         "config": {"workload": "block-sparse causal fwd bf16 B=2 H=16 S=16384 D=128, 64x64 blocks, band 8 + 4 sink + 10%% (%d live blocks)" % live,
                    "flop_per_step": flop,
                    "kv_tile_bytes_per_step": float(live * 64 * D * 2 * 2 * B * H),
@@ -280,12 +389,19 @@ def run_sparse_decode(steps, warmup):
     B, Hq, Hkv, L, D = 32, 32, 8, 131072, 128
     g = torch.Generator().manual_seed(1)
     lens = (L - torch.randint(0, 64, (B,), generator=g)).to(torch.int32)
-    idx = masks.synthetic_decode_blocks(B, Hkv, L // 64, 128, seed=2).cuda()
+    # Six seeded index lists, rotated: six steps read 6 x 1.08 GB of different blocks, so no step
+    # finds the blocks of an earlier one in the 256 MB last-level cache.
+    lists = [masks.synthetic_decode_blocks(B, Hkv, L // 64, 128, seed=2 + i).cuda() for i in range(6)]
+    idx = lists[0]
     lens_d = lens.cuda()
     q = _randn((B, Hq, D), 0)
     kc, vc = _randn((B, Hkv, L, D), 1), _randn((B, Hkv, L, D), 2)
-    fn = lambda: ta.flash_attention_sparse_decoding(q, kc.transpose(1, 2), vc.transpose(1, 2), None,
-                                                    seq_lens=lens_d, block_indices=idx)
+    state = {"i": 0}
+
+    def fn():
+        state["i"] += 1
+        return ta.flash_attention_sparse_decoding(q, kc.transpose(1, 2), vc.transpose(1, 2), None,
+                                                  seq_lens=lens_d, block_indices=lists[state["i"] % len(lists)])
     ms = _time_steps(fn, steps, warmup)
     from tritonops_amd import _lib
     lib = _lib.load()
@@ -306,21 +422,45 @@ def run_sparse_decode(steps, warmup):
     a.block_idx, a.block_cnt = idx.data_ptr(), None
     a.block_idx_stride_b, a.block_idx_stride_h = Hkv * 128, 128
     a.max_blocks, a.block_size = 128, 64
-    a.split_blocks = lib.mi_decode_choose_split_blocks(B, Hkv, 129, 256)
+    a.split_blocks = lib.mi_decode_choose_split_blocks(B, Hkv, 129, lib.mi_device_cu_count())
     a.window_local = a.window_global = -1
     a.include_last_block = 1
     nb = lib.mi_decode_workspace_bytes(C.byref(a))
     ws = torch.empty(nb, device="cuda", dtype=torch.uint8)
     a.workspace, a.workspace_bytes = ws.data_ptr(), nb
-    kms = _event_ms(3, a, steps, warmup)
+    rot = []
+    for l in lists:
+        ai = _lib.DecodeArgs.from_buffer_copy(a)
+        ai.block_idx = l.data_ptr()
+        rot.append(ai)
+    kms = _event_ms(3, rot, steps, warmup)
+    kms_one_list = _event_ms(3, a, steps, warmup)
     nbytes_alg = float(B * Hkv * 129 * 64 * D * 2 * 2)
+    # parity on the benchmark tensors: three sequences (first list) against fp32 torch math on the device
+    got = ta.flash_attention_sparse_decoding(q, k, v, None, seq_lens=lens_d, block_indices=idx)
+    err = 0.0
+    for b in (0, 15, 31):
+        n = int(lens[b])
+        blocks = torch.cat([idx[b].long(), torch.full((Hkv, 1), (n - 1) // 64, device="cuda")], 1)      # [Hkv, 129]
+        tok = (blocks[:, :, None] * 64 + torch.arange(64, device="cuda")).reshape(Hkv, -1)             # [Hkv, 129*64]
+        live = tok < n
+        tok = tok.clamp(max=n - 1)
+        kk = torch.gather(kc[b], 1, tok[:, :, None].expand(-1, -1, D)).float()
+        vv = torch.gather(vc[b], 1, tok[:, :, None].expand(-1, -1, D)).float()
+        sc = torch.einsum("gid,gld->gil", q[b].view(Hkv, Hq // Hkv, D).float(), kk) * D ** -0.5
+        sc = sc.masked_fill(~live[:, None, :], float("-inf"))
+        want = torch.einsum("gil,gld->gid", torch.softmax(sc, -1), vv).reshape(Hq, D)
+        err = max(err, _err(got[b], want))
     return {
         "name": "sparse_decode", "ms_per_step": ms, "kernel_ms": kms,
         "metric": "sparse_decode_hbm_gbs", "unit": "GB/s", "value": nbytes_alg / (ms * 1e-3) / 1e9,
+        "max_abs_err": err,
+        "err_sample": "3 of the 32 sequences (all heads, first index list) against fp32 torch math on the device",
         "roofline": {"bound": "hbm", "achieved": nbytes_alg / (kms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "kernel": "decode_splitkv_kernel<bf16,128> (block list)"},
+                     "unit": "GB/s", "kernel": KERNELS["sparse_decode"]},
         "config": {"workload": "block-sparse decode bf16 B=32 Hq=32 Hkv=8 KV=131072 D=128, top-128 of 64-token blocks + last block",
-                   "bytes_per_step": nbytes_alg, "split_blocks": int(a.split_blocks)},
+                   "bytes_per_step": nbytes_alg, "split_blocks": int(a.split_blocks),
+                   "index_lists_rotated": len(lists), "kernel_ms_same_list_every_launch": kms_one_list},
     }
 
 
@@ -352,11 +492,23 @@ def run_rmsnorm(steps, warmup):
     k_bwd = _event_ms(7, a, steps, warmup)
     b_fwd = 2.0 * T * D * 2 + T * 4                 # x read, y written, rsqrt written
     b_bwd = 3.0 * T * D * 2 + T * 4                 # x, dy read, dx written, rsqrt read
+    # parity on the benchmark tensors: 512 rows of y and dx, and dw over all rows, against fp32 torch math
+    rows = torch.arange(0, T, T // 512, device="cuda")
+    xf, dyf = x[rows].float(), dy[rows].float()
+    r = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    want_dx = dyf * w * r - xf * r.pow(3) * (dyf * w * xf).sum(-1, keepdim=True) / D
+    r_all = torch.rsqrt(x.float().pow(2).mean(-1, keepdim=True) + eps)
+    want_dw = (dy.float() * x.float() * r_all).sum(0)
+    err = max(_err(y[rows], xf * r * w), _err(dx[rows], want_dx))
+    err_dw = float(((dw.float() - want_dw).abs() / want_dw.abs().clamp(min=1.0)).max().item())
+    del r_all, want_dw
     return {
         "name": "rmsnorm", "ms_per_step": ms, "kernel_ms": k_fwd + k_bwd,
         "metric": "rmsnorm_fwd_bwd_hbm_gbs", "unit": "GB/s", "value": (b_fwd + b_bwd) / (ms * 1e-3) / 1e9,
+        "max_abs_err": err, "max_rel_err_dw": err_dw,
+        "err_sample": "y and dx of 512 of the 32768 rows, dw over all rows (relative), against fp32 torch math on the device",
         "roofline": {"bound": "hbm", "achieved": (b_fwd + b_bwd) / ((k_fwd + k_bwd) * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "kernel": "rms_fwd_vec_kernel + rms_bwd_vec_kernel + rms_dw_reduce_kernel"},
+                     "unit": "GB/s", "kernel": KERNELS["rmsnorm"]},
         "config": {"workload": "RMSNorm fwd + bwd, x [32768, 4096] bf16, weight fp32, eps 1e-6",
                    "bytes_per_step": b_fwd + b_bwd, "fwd_kernel_ms": k_fwd, "bwd_kernel_ms": k_bwd,
                    "fwd_gbs": b_fwd / (k_fwd * 1e-3) / 1e9, "bwd_gbs": b_bwd / (k_bwd * 1e-3) / 1e9},
@@ -396,11 +548,20 @@ def run_fused_xent(steps, warmup):
     kms_grad = _event_ms(10, g, max(steps // 2, 2), 1)
     del dl
     flop = 2.0 * T * D * N
+    # parity on the benchmark tensors: loss and lse of 64 tokens against fp32 torch math on the device
+    rows = torch.arange(0, T, T // 64, device="cuda")
+    logits = x[rows].float() @ w.float().t()
+    want_lse = torch.logsumexp(logits, -1)
+    want_loss = want_lse - logits.gather(-1, y[rows].view(-1, 1)).squeeze(-1)
+    err = max(_err(loss[rows], want_loss), _err(lse[rows], want_lse))
+    del logits
     return {
         "name": "fused_xent", "ms_per_step": ms, "kernel_ms": kms,
         "metric": "fused_linear_xent_fwd_tflops", "unit": "TFLOP/s", "value": flop / (ms * 1e-3) / 1e12,
+        "max_abs_err": err,
+        "err_sample": "loss and lse of 64 of the 8192 tokens against fp32 torch math on the device",
         "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "kernel": "xent_fwd_kernel<bf16> (+ combine)"},
+                     "unit": "TFLOP/s", "kernel": KERNELS["fused_xent"]},
         "config": {"workload": "fused linear + cross-entropy forward bf16, T=8192 tokens, hidden 4096, vocabulary 128256",
                    "flop_per_step": flop, "bwd_ms_per_step": ms_bwd, "dlogits_kernel_ms": kms_grad,
                    "bwd_note": "backward = the same GEMM kernel with the dlogits epilogue (dlogits_kernel_ms) + two "
@@ -411,6 +572,7 @@ def run_fused_xent(steps, warmup):
 
 WORKLOADS = {
     "dense_causal": run_dense_causal,
+    "c1_dense_noncausal_small": run_c1_small,
     "gqa_decode": run_decode,
     "block_sparse": run_block_sparse,
     "sparse_decode": run_sparse_decode,
@@ -445,6 +607,43 @@ def cpu_baseline(name):
         return {"value": flop / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
                 "sample": "torch-CPU bf16 causal softmax(qk^T/sqrt(d))v (tutorial/4.4 oracle) on B=1 H=16 S=8192 D=128 (1/8 of the workload), "
                           "median of 3; same algorithmic-FLOP formula as the GPU figure",
+                "seconds": t}
+    if name == "c1_dense_noncausal_small":
+        B, H, S, D = 1, 4, 256, 64
+        q, k, v = (torch.randn((B, H, S, D), generator=g) for _ in range(3))
+        t = med(lambda: orc.full_attention(q, k, v), reps=21)
+        flop = 4.0 * B * H * S * S * D
+        return {"value": flop / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "sample": "torch-CPU fp32 softmax(q k^T / sqrt(d)) v (tutorial/4.3.multi_head_attention.py:11-19) on the "
+                          "whole workload B=1 H=4 S=256 D=64, median of 21",
+                "seconds": t}
+    if name == "block_sparse":
+        from tritonops_amd import masks
+        B, H, S, D = 1, 2, 16384, 128
+        m = masks.synthetic_block_mask(S // 64, 8, 4, 0.10, seed=2)
+        live, nb = int(m.sum()), S // 64
+        q, k, v = (torch.randn((1, S, H, D), generator=g).to(torch.bfloat16) for _ in range(3))
+        cu = torch.tensor([0, S], dtype=torch.int32)
+        t = med(lambda: orc.block_sparse_attention(q, k, v, cu, m), reps=1)
+        flop = 4.0 * D * ((live - nb) * 64 * 64 + nb * 64 * 65 / 2) * B * H
+        return {"value": flop / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "sample": "torch-CPU bf16 masked softmax(q k^T scale) v under the same block mask (the math of "
+                          "flash_attn_sparse_attn_triton.py:391-442; it computes the full S x S scores and masks them) "
+                          "on B=1 H=2 of B=2 H=16 (1/16 of the workload), one timed run after a warm-up; same "
+                          "algorithmic-FLOP formula as the GPU figure (live blocks only)",
+                "seconds": t}
+    if name == "sparse_decode":
+        from tritonops_amd import masks
+        B, Hq, Hkv, L, D = 2, 32, 8, 131072, 128
+        lens = (L - torch.randint(0, 64, (B,), generator=g)).to(torch.int32)
+        idx = masks.synthetic_decode_blocks(B, Hkv, L // 64, 128, seed=2)
+        q = torch.randn((B, Hq, D), generator=g).to(torch.bfloat16)
+        k, v = (torch.randn((B, L, Hkv, D), generator=g, dtype=torch.bfloat16) for _ in range(2))
+        t = med(lambda: orc.block_sparse_decoding(q, k, v, lens, idx))
+        nb = float(B * Hkv * 129 * 64 * D * 2 * 2)
+        return {"value": nb / t / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+                "sample": "torch-CPU bf16 decode oracle (flash_attn_decoding_sparse.py:368-406 math under the block list) "
+                          "on B=2 of the 32 sequences, median of 3; same algorithmic-byte formula as the GPU figure",
                 "seconds": t}
     if name == "gqa_decode":
         B, Hq, Hkv, L, D = 8, 32, 8, 32768, 128
@@ -541,7 +740,13 @@ def main():
         r = WORKLOADS[n](a.steps, a.warmup)
         rf = r["roofline"]
         rf["frac"] = rf["achieved"] / rf["peak"]
-        rf["traffic"] = traffic.get(r["name"], {}).get("hbm_bytes_per_launch")
+        # HBM bytes per launch from the committed rocprofv3 counter runs; only a reading taken from the
+        # kernels this workload launches today is reported
+        t = traffic.get(r["name"], {})
+        fresh = t.get("kernel") == rf["kernel"]
+        rf["traffic"] = t.get("hbm_bytes_per_launch") if fresh else None
+        rf["traffic_source"] = ("profiles/hbm_traffic.json, measured at commit %s" % traffic.get("_commit", "?")
+                                if fresh else "no counter run of this kernel on file")
         results.append(r)
         torch.cuda.empty_cache()
     head = results[0]
@@ -551,7 +756,9 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic N(0,1) inputs drawn from a seed, resident in HBM",
         "config": head["config"], "roofline": head["roofline"], "kernel_ms": head["kernel_ms"],
+        "max_abs_err": head.get("max_abs_err"), "err_sample": head.get("err_sample"),
         "device": torch.cuda.get_device_name(0),
+        "compute_units": torch.cuda.get_device_properties(0).multi_processor_count,
     }
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(head["name"])
@@ -559,7 +766,8 @@ def main():
             out["cpu_baseline"]["host_cpus"] = os.cpu_count()
     if len(results) > 1:
         out["other_workloads"] = [
-            {k: r[k] for k in ("name", "metric", "value", "unit", "ms_per_step", "kernel_ms", "roofline", "config")}
+            {k: r[k] for k in ("name", "metric", "value", "unit", "ms_per_step", "kernel_ms", "max_abs_err",
+                               "err_sample", "roofline", "config") if k in r}
             for r in results[1:]]
         if not a.no_cpu_baseline:
             for r in out["other_workloads"]:

@@ -476,3 +476,18 @@ def test_product_package_never_imports_the_oracle():
             if f.endswith((".py", ".cpp", ".hip", ".h")):
                 text = open(os.path.join(dirpath, f), encoding="utf-8", errors="ignore").read()
                 assert not pat.search(text), os.path.join(dirpath, f)
+
+
+def test_bench_names_kernels_that_exist_in_the_library():
+    """bench.py reports, per workload, the device symbol its roofline figure is
+    about; every such symbol must be in the built library."""
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("bench", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    blob = open(_lib.LIB_PATH, "rb").read()
+    assert set(bench.KERNELS) == set(bench.WORKLOADS)
+    for workload, names in bench.KERNELS.items():
+        for name in names.split(" + "):
+            assert name.encode() in blob, (workload, name)
