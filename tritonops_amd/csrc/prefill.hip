@@ -392,6 +392,10 @@ dense_kernel(const PrefillParams p) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // 32-row block of the item that this wave owns.  Waves w and w + 4 share a
+  // SIMD; in the diagonal block of a causal item row block r has r + 1 halves
+  // to do, so pairing blocks (r, 7 - r) gives every SIMD the same nine.
+  const int rblk = wave < 4 ? wave : 11 - wave;
   F fr;
   fr.init(lane, (uint32_t)(uintptr_t)smem, VBASE);
   DMA dma;
@@ -436,7 +440,7 @@ dense_kernel(const PrefillParams p) {
   // Q^T operands of an item (lane (query lq, half lh) holds d = 16c + 8lh .. +7)
   // and its first NS-1 tiles; nothing waits here
   auto request_item = [&](const Item& it, i32x4 (&Q)[G::KSTEPS]) __attribute__((always_inline)) {
-    const int row = min(it.q0 + 32 * wave + fr.lq, it.len - 1);
+    const int row = min(it.q0 + 32 * rblk + fr.lq, it.len - 1);
     const T* qr = it.qp + (int64_t)row * p.q_ss + 8 * fr.lh;
     // Issued from inline assembly like the tile loads, and for the same reason:
     // a load the compiler knows about is guarded by a counted wait at its first
@@ -455,7 +459,9 @@ dense_kernel(const PrefillParams p) {
   i32x4 Qf[G::KSTEPS];
   f32x16 O[G::NDB];
   float m, l;
+  float m_neg;  // -m, or 0 while m is still -inf: the addend of every exponent (changes only in exact_fix)
   int len, n_tiles, q0w, qrow, row_lim, H_w;
+  int tail_t;  // first tile (> 0) at whose top no further tile is requested
   f32x16 S[2];
   constexpr int KR = G::KSTEPS < 4 ? G::KSTEPS : 4;  // K fragments kept in flight
   i32x4 kf[KR];  // fragments 0..KR-1 of the half that is scored next, read one block ahead
@@ -486,7 +492,7 @@ dense_kernel(const PrefillParams p) {
   };
   auto exp_second = [&](int i, uint32_t (&Pd)[8], float& rs) __attribute__((always_inline)) {
     const float p1 = fast_exp2(e_u1);
-    rs += e_p0 + p1;
+    rs = i == 0 ? e_p0 + p1 : rs + (e_p0 + p1);  // pair 0 opens the row sum of its half
     Pd[i] = Elem<T>::pack2(e_p0, p1);
   };
   // rare: bring m to the exact running maximum including the half in Sx,
@@ -503,6 +509,7 @@ dense_kernel(const PrefillParams p) {
 #pragma unroll
     for (int db = 0; db < G::NDB; ++db) O[db] *= alpha;
     m = m_new;
+    m_neg = -m_safe;
     rs = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -533,7 +540,6 @@ dense_kernel(const PrefillParams p) {
     f32x16& Sn = S[KB ^ 1];
     uint32_t (&Pc)[8] = Pb[KB];
     uint32_t (&Pn)[8] = Pb[KB ^ 1];
-    const float m_neg = (m == -INFINITY) ? 0.f : -m;
     // Block A carries the serial chain of the eight S MFMAs: a raised issue
     // priority while a wave is in it (and a lower one in block B, whose MFMAs
     // form four independent chains) lets the two waves of a SIMD fall out of
@@ -560,9 +566,7 @@ dense_kernel(const PrefillParams p) {
     if (__builtin_amdgcn_ballot_w64(!(rsv[KB] <= kRowSumLimit)) != 0) exact_fix(Sc, Pc, rsv[KB]);
     l += rsv[KB];
     mask_half(h + 1, Sn);
-    const float m_neg2 = (m == -INFINITY) ? 0.f : -m;
     __builtin_amdgcn_s_setprio(1);
-    rsv[KB ^ 1] = 0.f;
 #pragma unroll
     for (int sl = 0; sl < 8; ++sl) {
       if (sl < 2 * G::NDB) {
@@ -574,7 +578,7 @@ dense_kernel(const PrefillParams p) {
       if (sl >= 4 && sl - 4 < KR) kf[sl - 4] = fr.load_k(K2OFF, KB, sl - 4);
       // (for the last half of a wave Sn holds scores of stale LDS contents: the results are never used)
       if ((sl & 1) == 0)
-        exp_first(Sn, sl / 2, m_neg2);
+        exp_first(Sn, sl / 2, m_neg);
       else
         exp_second(sl / 2, Pn, rsv[KB ^ 1]);
       __builtin_amdgcn_sched_barrier(0);
@@ -586,14 +590,20 @@ dense_kernel(const PrefillParams p) {
   // (Tile 0: the item's first barrier has done all of that.)
   auto tile_iter = [&](auto ts_c, int t) __attribute__((always_inline)) {
     constexpr int TS = decltype(ts_c)::value;
-    if (t > 0) {
-      // tile t+1 was requested NS-2 iterations ago; at most NS-3 younger tiles may still fly
-      if (t + NS - 2 < n_tiles)
+    if (t + NS - 1 < n_tiles) {
+      if (t > 0) {
+        // tile t+1 was requested NS-2 iterations ago; the younger tile t+2 may still fly
         __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 3) * 2 * IPW));
-      else
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+        __syncthreads();
+        dma.template tile<(TS + NS - 1) % NS>(cur.kv, (t + NS - 1) * TN);
+      }
+    } else if (t == tail_t) {
+      // Nothing is left to request: every remaining tile is in the ring or on
+      // its way.  One full wait and one barrier publish them all, and the waves
+      // then run to the end of the item without meeting again - in the diagonal
+      // block of a causal item each wave has its own number of halves to do.
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
       __syncthreads();
-      if (t + NS - 1 < n_tiles) dma.template tile<(TS + NS - 1) % NS>(cur.kv, (t + NS - 1) * TN);
     }
     half_step(ic<2 * TS>{}, 2 * t);
     half_step(ic<2 * TS + 1>{}, 2 * t + 1);
@@ -648,7 +658,14 @@ dense_kernel(const PrefillParams p) {
         const int och = ps * CH + ch;  // chunk of the output row
         if (och < G::NCH && q0w + row < len) {
           const i32x4 val = *reinterpret_cast<const i32x4*>(stage + row * SROW + ((ch ^ sswz(row)) << 4));
-          *reinterpret_cast<i32x4*>(cur.op + (int64_t)(q0w + row) * p.o_ss + och * 8) = val;
+          // One store instruction per statement, whatever the compiler would
+          // have made of a plain assignment: the wait at the top of the next
+          // item counts on exactly kOutStores of them behind the loads that
+          // request_item() issued.  The s_nop covers the wait states a store
+          // of more than 8 bytes needs before its data registers may be
+          // overwritten (the compiler pads its own stores, not this one).
+          T* dst = cur.op + (int64_t)(q0w + row) * p.o_ss + och * 8;
+          asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1" : : "v"(dst), "v"(val) : "memory");
         }
       }
       asm volatile("" ::: "memory");
@@ -661,16 +678,18 @@ dense_kernel(const PrefillParams p) {
   while (have) {
     len = cur.len;
     n_tiles = cur.n_tiles;
-    q0w = cur.q0 + 32 * wave;
+    q0w = cur.q0 + 32 * rblk;
     qrow = q0w + fr.lq;
     row_lim = causal ? min(qrow, len - 1) : len - 1;  // largest key this lane may see
     H_w = (len + 31) / 32;                            // halves this wave works on
     if (causal) H_w = min(H_w, q0w / 32 + 1);         // nothing above its own diagonal block
     H_w = min(H_w, 2 * n_tiles);
     if (q0w >= len) H_w = 0;                          // all rows past the sequence end
+    tail_t = max(1, n_tiles - (NS - 1));
 #pragma unroll
     for (int db = 0; db < G::NDB; ++db) O[db] = (f32x16){0};
     m = -INFINITY;
+    m_neg = 0.f;
     l = 0.f;
 
     // Every load requested so far must have landed: the Q operands and tile 0
@@ -686,6 +705,11 @@ dense_kernel(const PrefillParams p) {
       __builtin_amdgcn_s_waitcnt(waitcnt_vm(kOutStores));
     else
       __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    // The Q registers were written by loads the compiler cannot see.  Passing
+    // them through an empty statement HERE makes every use of them depend on a
+    // point behind the wait, so no read of them can be scheduled above it.
+#pragma unroll
+    for (int c = 0; c < G::KSTEPS; ++c) asm volatile("" : "+v"(Qf[c]));
     __syncthreads();
     if (NS - 1 < n_tiles) dma.template tile<NS - 1>(cur.kv, (NS - 1) * TN);
     if (H_w > 0) {
@@ -697,10 +721,9 @@ dense_kernel(const PrefillParams p) {
       S[0] = acc;
       mask_half(0, S[0]);
       exact_fix(S[0], Pb[0], rsv[0]);
-      rsv[0] = 0.f;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        exp_first(S[0], i, (m == -INFINITY) ? 0.f : -m);
+        exp_first(S[0], i, m_neg);
         exp_second(i, Pb[0], rsv[0]);
       }
 #pragma unroll
