@@ -263,6 +263,13 @@ def test_backward_and_rmsnorm_validation(lib):
     assert lib.mi_attn_bwd_validate(C.byref(a)) == 0
     a.dk = None
     assert lib.mi_status_name(lib.mi_attn_bwd_validate(C.byref(a))).decode() == "MI_ERR_NULL_POINTER"
+    a.dk = 0x1000
+    for field in ("q_stride_s", "dout_stride_s", "lse_stride_s"):      # streamed tiles use 32-bit lane offsets
+        for bad in (-1024, 1 << 24):
+            setattr(a, field, bad)
+            assert lib.mi_status_name(lib.mi_attn_bwd_validate(C.byref(a))).decode() == "MI_ERR_STRIDE", field
+        setattr(a, field, 1024)
+    assert lib.mi_attn_bwd_validate(C.byref(a)) == 0
     a.dk, a.heads_kv = 0x1000, 3
     assert lib.mi_status_name(lib.mi_attn_bwd_validate(C.byref(a))).decode() == "MI_ERR_GQA"
     a.heads_kv, a.struct_size = 2, 8

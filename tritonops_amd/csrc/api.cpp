@@ -339,6 +339,11 @@ int mi_attn_bwd_validate(const mi_attn_bwd_args* a) {
                         a->dq_stride_h, a->dk_stride_s, a->dk_stride_h, a->dv_stride_s, a->dv_stride_h};
   for (int64_t x : st)
     if (!mult8(x)) return fail(MI_ERR_STRIDE, "tensor strides must be multiples of 8 elements (got %lld)", (long long)x);
+  // a streamed 64-row tile is addressed as uniform base + 32-bit byte offset per lane
+  const int64_t ss[] = {a->q_stride_s, a->k_stride_s, a->v_stride_s, a->dout_stride_s, a->lse_stride_s};
+  for (int64_t x : ss)
+    if (x < 0 || x >= (1 << 24))
+      return fail(MI_ERR_STRIDE, "q/k/v/dout/lse sequence strides must be in [0, 2^24) elements (got %lld)", (long long)x);
   if (!a->cu_seqlens) {
     const int64_t sb[] = {a->q_stride_b, a->k_stride_b, a->v_stride_b, a->o_stride_b, a->dout_stride_b,
                           a->dq_stride_b, a->dk_stride_b, a->dv_stride_b};

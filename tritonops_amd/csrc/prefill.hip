@@ -245,10 +245,24 @@ sparse_kernel(const PrefillParams p) {
   const int beg = __builtin_amdgcn_readfirstlane(rp[qt]);
   const int n_tiles = __builtin_amdgcn_readfirstlane(rp[qt + 1] - beg) * (kTileN / TN);
   const int32_t* cols = p.col_idx + g.b * p.ci_sb + h * p.ci_sh + beg;
-  // first key of tile `it`
+  // The block list is kept in registers, 64 entries at a time (lane l holds
+  // entry 64 * chunk + l; the chunk being walked and the one behind it), and
+  // read with v_readlane.  A memory load inside the tile loop would have to be
+  // waited for with vmcnt(0), which also drains the tile that was requested a
+  // moment ago: the ring would never have a load in flight during a compute.
+  const int n_blk = n_tiles / (kTileN / TN);
+  auto load_cols = [&](int chunk) __attribute__((always_inline)) -> int {
+    const int idx = chunk * 64 + lane;
+    return idx < n_blk ? cols[idx] : 0;
+  };
+  int col_chunk = 0;
+  int col_cur = load_cols(0), col_nxt = load_cols(1);
+  // first key of tile `it` (it lies in the chunk being walked or in the next one)
   auto tile_k0 = [&](int it) __attribute__((always_inline)) -> int {
     constexpr int PER = kTileN / TN;
-    return __builtin_amdgcn_readfirstlane(cols[it / PER]) * kTileN + (it % PER) * TN;
+    const int q = it / PER;
+    const int v = (q >> 6) == col_chunk ? col_cur : col_nxt;
+    return __builtin_amdgcn_readlane(v, q & 63) * kTileN + (it % PER) * TN;
   };
 
   // ---- Q^T operands: lane (query lq, half lh) holds d = 16c + 8lh .. +7
@@ -266,6 +280,11 @@ sparse_kernel(const PrefillParams p) {
 
   auto step = [&](auto stage_c, int it) {
     constexpr int ST = decltype(stage_c)::value;
+    if (((it / (kTileN / TN)) >> 6) != col_chunk) {  // walked into the next 64 entries of the list
+      ++col_chunk;
+      col_cur = col_nxt;
+      col_nxt = load_cols(col_chunk + 1);
+    }
     // refill the stage that was read in the previous iteration
     const bool refill = it + NS - 1 < n_tiles;
     if (refill) dma.template tile<(ST + NS - 1) % NS>(kv, tile_k0(it + NS - 1));
