@@ -136,6 +136,16 @@ struct TileDma {
                  : "memory");
   }
 
+  // The same with the address as "uniform 64-bit base + 32-bit lane offset"
+  // (no vector arithmetic per load).
+  static __device__ __forceinline__ void dma16s(uint64_t base, uint32_t off, uint32_t slab_u) {
+    const uint32_t slab = (uint32_t)__builtin_amdgcn_readfirstlane(slab_u);
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(off), "s"(base), "s"(slab)
+                 : "memory");
+  }
+
   __device__ __forceinline__ void init(const PrefillParams& p, int lane_, int wave_) {
     lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem);
     wave = wave_;
@@ -180,14 +190,23 @@ struct TileDma {
     if (k0 + TN <= s.len) {
       // whole tile inside the sequence
       const uint32_t k0u = (uint32_t)__builtin_amdgcn_readfirstlane(k0);
+      // (scalar base + lane offset pays in the dense kernel; the block-sparse one,
+      // whose base changes with every listed block, measured faster with the sum in vector registers)
+      constexpr bool kScalarBase = NW >= 8;
       const uint64_t kt_u = s.k_base + (uint64_t)k0u * k_pitch, vt_u = s.v_base + (uint64_t)k0u * v_pitch;
+      const uint64_t kt_s = kScalarBase ? uniform64(kt_u) : 0, vt_s = kScalarBase ? uniform64(vt_u) : 0;
 #pragma unroll
       for (int t = 0; t < IPW; ++t) {
         const int inst = wave + NW * t;
         const int r = RPI * inst + drow;
         const int kc = dslot ^ F::swz_k(r), vc = dslot ^ F::swz_v(r);
-        if (D != 96 || kc < G::NCH) dma16(reinterpret_cast<const char*>(kt_u + koff[t]), sK + inst * 1024);
-        if (D != 96 || vc < G::NCH) dma16(reinterpret_cast<const char*>(vt_u + voff[t]), sV + inst * 1024);
+        if (kScalarBase) {
+          if (D != 96 || kc < G::NCH) dma16s(kt_s, koff[t], sK + inst * 1024);
+          if (D != 96 || vc < G::NCH) dma16s(vt_s, voff[t], sV + inst * 1024);
+        } else {
+          if (D != 96 || kc < G::NCH) dma16(reinterpret_cast<const char*>(kt_u + koff[t]), sK + inst * 1024);
+          if (D != 96 || vc < G::NCH) dma16(reinterpret_cast<const char*>(vt_u + voff[t]), sV + inst * 1024);
+        }
       }
     } else {
       // rows past the sequence end re-read its last row (masked later)
