@@ -38,6 +38,15 @@ namespace {
 template <int V>
 using ic = std::integral_constant<int, V>;
 
+// f(ic<B>{}), f(ic<B + 1>{}), ..., f(ic<E - 1>{})
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (B < E) {
+    f(ic<B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+
 // vmcnt(N) expcnt(7) lgkmcnt(15) for s_waitcnt on gfx9-family encodings
 constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
 // vmcnt(63) expcnt(7) lgkmcnt(N)
@@ -497,87 +506,128 @@ __device__ __forceinline__ void bwd_dkdv_item(const BwdParams& p, const int bid,
   const int n_stream = nj * gqa;
 
   const int drow = lane / F::SLOTS, dslot = lane % F::SLOTS;
-  auto dma16 = [&](const char* g, uint32_t slab_u) __attribute__((always_inline)) {
-    const uint32_t slab = (uint32_t)__builtin_amdgcn_readfirstlane(slab_u);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(slab) : "memory");
-  };
-  auto dma4 = [&](const char* g, uint32_t slab_u) __attribute__((always_inline)) {
-    const uint32_t slab = (uint32_t)__builtin_amdgcn_readfirstlane(slab_u);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" : : "v"(g), "s"(slab) : "memory");
-  };
-  auto dma16s = [&](uint64_t base, uint32_t off, uint32_t slab_u) __attribute__((always_inline)) {
-    const uint32_t slab = (uint32_t)__builtin_amdgcn_readfirstlane(slab_u);
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"(base), "s"(slab) : "memory");
-  };
-  auto dma4s = [&](uint64_t base, uint32_t off, uint32_t slab_u) __attribute__((always_inline)) {
-    const uint32_t slab = (uint32_t)__builtin_amdgcn_readfirstlane(slab_u);
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" : : "v"(off), "s"(base), "s"(slab) : "memory");
-  };
   auto uniform64 = [](uint64_t x) __attribute__((always_inline)) -> uint64_t {
     const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)x);
     const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(x >> 32));
     return ((uint64_t)hi << 32) | lo;
   };
-  // streamed tensors of the first query head of the group, first row of the sequence
+  // A direct-to-LDS load of the lanes in `mask` (all 64 lanes are active and
+  // control flow is wave-uniform wherever this is called, so exec is restored
+  // to all ones).  Switching a load off through the exec mask keeps it in
+  // straight-line code: a branch around it would end the basic block and let
+  // the compiler move the arithmetic that is meant to sit behind the MFMAs.
+  auto dma_masked = [&](uint64_t mask, uint64_t base, uint32_t off, uint32_t slab, auto wide_c) __attribute__((always_inline)) {
+    if (decltype(wide_c)::value)
+      asm volatile("s_mov_b32 m0, %3\n\ts_mov_b64 exec, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, -1"
+                   : : "s"(mask), "v"(off), "s"(base), "s"(slab) : "memory");
+    else
+      asm volatile("s_mov_b32 m0, %3\n\ts_mov_b64 exec, %0\n\tglobal_load_lds_dword %1, %2\n\ts_mov_b64 exec, -1"
+                   : : "s"(mask), "v"(off), "s"(base), "s"(slab) : "memory");
+  };
+
+  // ---- streamed tiles.  Per tile and wavefront: four loads of 1 KiB (two of
+  // Q, two of dO); wavefronts 0 and 1 also fetch the tile's 64 lse / Delta
+  // values.  The addresses are running, wave-uniform values: they advance by
+  // one tile per request and jump to the next query head of the group when a
+  // head's tiles are through (one add each per step; the item's scalar
+  // bookkeeping is issued by the same wavefronts that feed the MFMAs, one
+  // instruction per four cycles, so every instruction saved per step counts).
   const int64_t pitch0 = p.q_ss * 2, pitch1 = p.do_ss * 2;
-  const char* h0 = reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.q) + bsel * p.q_sb + start * p.q_ss + hr * gqa * p.q_sh);
-  const char* h1 = reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.dout) + bsel * p.do_sb + start * p.do_ss + hr * gqa * p.do_sh);
-  const char* lv0 = reinterpret_cast<const char*>(p.lse + bsel * p.lse_sb + start * p.lse_ss + hr * gqa * p.lse_sh);
-  const char* dv0 = reinterpret_cast<const char*>(p.delta + (int64_t)b * p.dl_sb + (int64_t)hr * gqa * p.dl_sh);
+  const char* h0 = reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.q) + bsel * p.q_sb + (start + j0 * TN) * p.q_ss + hr * gqa * p.q_sh);
+  const char* h1 = reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.dout) + bsel * p.do_sb + (start + j0 * TN) * p.do_ss + hr * gqa * p.do_sh);
+  const char* hl = wave == 0
+      ? reinterpret_cast<const char*>(p.lse + bsel * p.lse_sb + (start + j0 * TN) * p.lse_ss + hr * gqa * p.lse_sh)
+      : reinterpret_cast<const char*>(p.delta + (int64_t)b * p.dl_sb + (int64_t)hr * gqa * p.dl_sh + j0 * TN);
+  const int64_t pitchl = wave == 0 ? p.lse_ss * 4 : 4;
+  uint64_t a0 = uniform64((uint64_t)(uintptr_t)h0), a1 = uniform64((uint64_t)(uintptr_t)h1), al = uniform64((uint64_t)(uintptr_t)hl);
+  const uint64_t step0 = uniform64((uint64_t)(TN * pitch0)), step1 = uniform64((uint64_t)(TN * pitch1));
+  const uint64_t stepl = uniform64((uint64_t)(TN * pitchl));
+  const uint64_t wrap0 = uniform64((uint64_t)(p.q_sh * 2 - (int64_t)(nj - 1) * TN * pitch0));
+  const uint64_t wrap1 = uniform64((uint64_t)(p.do_sh * 2 - (int64_t)(nj - 1) * TN * pitch1));
+  const uint64_t wrapl = uniform64((uint64_t)((wave == 0 ? p.lse_sh * 4 : p.dl_sh * 4) - (int64_t)(nj - 1) * TN * pitchl));
   uint32_t off0[IPW], off1[IPW];
+  uint64_t lane_mask[IPW];
 #pragma unroll
   for (int t = 0; t < IPW; ++t) {
     const int r = RPI * (wave + NW * t) + drow;
     const int c = dslot ^ F::swz(r);
     off0[t] = (uint32_t)r * (uint32_t)pitch0 + c * 16;
     off1[t] = (uint32_t)r * (uint32_t)pitch1 + c * 16;
+    lane_mask[t] = __builtin_amdgcn_ballot_w64(G::NCH == 16 || c < G::NCH);
   }
-  const uint32_t lv_off = (uint32_t)lane * (uint32_t)(p.lse_ss * 4);
-  // streamed tiles are requested in order: (head, tile, stage) of the next
-  // request; Q rows, dO rows, lse and Delta of the rows
-  int iss_g = 0, iss_j = j0, iss_st = 0;
-  auto issue = [&]() __attribute__((always_inline)) {
-    const int s0 = iss_j * TN;
-    const uint32_t base = lds0 + (uint32_t)iss_st * STAGEB;
-    const char* t0 = h0 + iss_g * (p.q_sh * 2);
-    const char* t1 = h1 + iss_g * (p.do_sh * 2);
-    const char* lp = lv0 + iss_g * (p.lse_sh * 4);
-    const char* dp = dv0 + (int64_t)iss_g * p.dl_sh * 4;
-    if (s0 + TN <= len) {
-      const uint64_t a0 = uniform64((uint64_t)(uintptr_t)(t0 + s0 * pitch0));
-      const uint64_t a1 = uniform64((uint64_t)(uintptr_t)(t1 + s0 * pitch1));
-#pragma unroll
-      for (int t = 0; t < IPW; ++t) {
-        const int inst = wave + NW * t;
-        const int c = dslot ^ F::swz(RPI * inst + drow);
-        if (G::NCH == 16 || c < G::NCH) {
-          dma16s(a0, off0[t], base + inst * 1024);
-          dma16s(a1, off1[t], base + TILEB + inst * 1024);
-        }
-      }
-      if (wave == 0) dma4s(uniform64((uint64_t)(uintptr_t)(lp + s0 * (p.lse_ss * 4))), lv_off, base + 2 * TILEB);
-      if (wave == 1) dma4s(uniform64((uint64_t)(uintptr_t)(dp + s0 * 4)), (uint32_t)lane * 4u, base + 2 * TILEB + 256);
+  const uint32_t lv_off = (uint32_t)lane * (uint32_t)pitchl;
+  const uint64_t lv_mask = wave < 2 ? ~0ull : 0ull;
+  constexpr int kDrips = 2 * IPW;
+  static_assert(kDrips == 4, "compute() places four loads");
+  int iss_left = nj;        // tiles of the current head still to request
+  int iss_s0 = j0 * TN;     // first row of the next request
+  int iss_st = 0;           // its stage
+  uint32_t iss_base = lds0; // and the stage's LDS address
+  uint64_t drip_on = 0;     // all ones while the loads of a request are still to be sent by compute()
+  // request(): a tile that reaches past the sequence end is loaded at once,
+  // row by row with clamped row numbers (masked later); a full tile only arms
+  // drip(), and compute() sends the four loads between its MFMAs: eight
+  // wavefronts that send their loads together right after the barrier stand
+  // in the memory pipeline's queue before any of them starts its arithmetic.
+  auto request = [&]() __attribute__((always_inline)) {
+    if (iss_s0 + TN <= len) {
+      drip_on = ~0ull;
     } else {
+      drip_on = 0;
+      const int last = len - 1 - iss_s0;  // >= 0
 #pragma unroll
       for (int t = 0; t < IPW; ++t) {
         const int inst = wave + NW * t;
         const int r = RPI * inst + drow;
         const int c = dslot ^ F::swz(r);
-        const int64_t rr = min(s0 + r, len - 1);  // rows past the end re-read the last row (masked later)
+        const int64_t rr = min(r, last);
+        const uint32_t slab = (uint32_t)__builtin_amdgcn_readfirstlane(iss_base + inst * 1024);
         if (G::NCH == 16 || c < G::NCH) {
-          dma16(t0 + rr * pitch0 + c * 16, base + inst * 1024);
-          dma16(t1 + rr * pitch1 + c * 16, base + TILEB + inst * 1024);
+          asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                       : : "v"((const char*)a0 + rr * pitch0 + c * 16), "s"(slab) : "memory");
+          asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                       : : "v"((const char*)a1 + rr * pitch1 + c * 16), "s"(slab + TILEB) : "memory");
         }
       }
-      const int64_t rr = min(s0 + lane, len - 1);
-      if (wave == 0) dma4(lp + rr * (p.lse_ss * 4), base + 2 * TILEB);
-      if (wave == 1) dma4(dp + rr * 4, base + 2 * TILEB + 256);
+      if (wave < 2) {
+        const int64_t rr = min(lane, last);
+        const uint32_t slab = (uint32_t)__builtin_amdgcn_readfirstlane(iss_base + 2 * TILEB + (wave == 0 ? 0 : 256));
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
+                     : : "v"((const char*)al + rr * pitchl), "s"(slab) : "memory");
+      }
     }
-    if (++iss_j == j0 + nj) {
-      iss_j = j0;
-      ++iss_g;
+  };
+  auto drip = [&](int k) __attribute__((always_inline)) {
+    const int t = k >> 1;
+    const int inst = wave + NW * t;
+    if (k & 1)
+      dma_masked(drip_on & lane_mask[t], a1, off1[t], iss_base + TILEB + inst * 1024, ic<1>{});
+    else
+      dma_masked(drip_on & lane_mask[t], a0, off0[t], iss_base + inst * 1024, ic<1>{});
+    if (k == 0) dma_masked(drip_on & lv_mask, al, lv_off, iss_base + 2 * TILEB + (wave == 0 ? 0 : 256), ic<0>{});
+  };
+  auto drip_all = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int k = 0; k < kDrips; ++k) drip(k);
+  };
+  // after the loads of a request are out: the next request's addresses
+  auto advance = [&]() __attribute__((always_inline)) {
+    drip_on = 0;
+    if (--iss_left == 0) {
+      iss_left = nj;
+      iss_s0 = j0 * TN;
+      a0 += wrap0;
+      a1 += wrap1;
+      al += wrapl;
+    } else {
+      iss_s0 += TN;
+      a0 += step0;
+      a1 += step1;
+      al += stepl;
     }
-    iss_st = iss_st == NS - 1 ? 0 : iss_st + 1;
+    const bool last_st = iss_st == NS - 1;
+    iss_st = last_st ? 0 : iss_st + 1;
+    iss_base = last_st ? lds0 : iss_base + STAGEB;
   };
 
   const float scale = p.scale;
@@ -586,19 +636,189 @@ __device__ __forceinline__ void bwd_dkdv_item(const BwdParams& p, const int bid,
   typedef float f32x4 __attribute__((ext_vector_type(4)));
   typedef __attribute__((address_space(3))) const f32x4 lds_f4;
 
-  // One streamed tile for this wave's role.  Both roles walk the same blocks.
-  int cmp_j = j0, cmp_slot = 0;  // tile and P slot of this wave's next compute() call
-  // (role and stage are compile-time: every LDS address below is a lane register plus an immediate)
-  auto compute = [&](auto role_c, auto stage_c) __attribute__((always_inline)) {
+  // ---- this wave's view of the tile it works on: LDS addresses that move
+  // from stage to stage (one add per address register and step, every read
+  // then is "register + immediate"; absolute stage offsets exceed the 16-bit
+  // immediate of an LDS instruction)
+  {
+    const uint32_t tro = grad ? TILEB : 0;   // tile read as row fragments: dO (grad) / Q (score)
+    const uint32_t tto = grad ? 0 : TILEB;   // tile read transposed for the accumulating product
+#pragma unroll
+    for (int c = 0; c < G::KSTEPS; ++c) fr.r_a[c] += tro;
+#pragma unroll
+    for (int db = 0; db < G::NDB; ++db) {
+      fr.t_a[db][0] += tto;
+      fr.t_a[db][1] += tto;
+    }
+  }
+  uint32_t lva = lds0 + 2 * TILEB + (grad ? 256u : 0u) + 8 * fr.lh * 4;   // lse (score) / Delta (grad) of the tile's rows
+  uint32_t pbv = lds0 + PBUF + (uint32_t)pr * 4096 + (uint32_t)lane * 16;   // P exchange slot of this 32-row group
+  int pb_step = (int)PSLOT;
+  int cmp_st = 0, cmp_left = nj, cmp_s0 = j0 * TN;
+  const bool rows_full = r0w + 32 <= len;
+  auto rotate = [&]() __attribute__((always_inline)) {
+    const bool last_st = cmp_st == NS - 1;
+    const int d = last_st ? -(NS - 1) * STAGEB : STAGEB;
+    cmp_st = last_st ? 0 : cmp_st + 1;
+#pragma unroll
+    for (int c = 0; c < G::KSTEPS; ++c) fr.r_a[c] += d;
+#pragma unroll
+    for (int db = 0; db < G::NDB; ++db) {
+      fr.t_a[db][0] += d;
+      fr.t_a[db][1] += d;
+    }
+    lva += d;
+    pbv += pb_step;
+    pb_step = -pb_step;
+    if (--cmp_left == 0) {
+      cmp_left = nj;
+      cmp_s0 = j0 * TN;
+    } else {
+      cmp_s0 += TN;
+    }
+  };
+
+  constexpr int kPrefetch = 4;
+  constexpr int NACC = 2 * G::NDB;
+  // One streamed tile for this wave's role, common case: all 64 streamed rows
+  // and all 32 resident rows exist and no pair is masked.  The two 32-row
+  // blocks of the tile are worked on as one software pipeline, so that the
+  // wave's vector arithmetic sits behind its own MFMAs:
+  //   1. chain(0)                          3. accumulate(0)  + arithmetic(1)
+  //   2. chain(1)  + arithmetic(0)         4. accumulate(1)
+  auto compute_fast = [&](auto role_c) __attribute__((always_inline)) {
     constexpr bool grad = decltype(role_c)::value != 0;
-    constexpr uint32_t stage = decltype(stage_c)::value * STAGEB;
-    constexpr uint32_t T0 = stage, T1 = stage + TILEB, LV = stage + 2 * TILEB;
-    const uint32_t pb = lds0 + PBUF + (uint32_t)cmp_slot * PSLOT + (uint32_t)pr * 4096 + (uint32_t)lane * 16;
-    const int s0 = cmp_j * TN;
-    if (++cmp_j == j0 + nj) cmp_j = j0;
-    cmp_slot ^= 1;
-    constexpr int kPrefetch = 4;
-    constexpr int NACC = 2 * G::NDB;
+    {
+      // Slots of the pipeline: phase 1 is slots 0 .. K-1, phase 2 K .. 2K-1,
+      // phase 3 2K .. 2K+NACC-1.  Pair i of block 0 is formed in phase 2,
+      // pair j of block 1 in phase 3; the lse / Delta values (four per LDS
+      // read) and the packed P a pair needs are read two slots earlier, so
+      // that only a few of them are live at a time (registers).
+      constexpr int K = G::KSTEPS;
+      auto slice_of = [](int i, int n) constexpr { int st = 0; while ((st + 1) * 8 / n <= i) ++st; return st; };
+      auto use_slot = [&](int sb, int i) constexpr { return sb == 0 ? K + slice_of(i, K) : 2 * K + slice_of(i, NACC); };
+      float lv[2][16];
+      i32x4 pp[2][2];  // grad wave: packed P of the two blocks
+      auto load_lv = [&](int sb, int q) __attribute__((always_inline)) {
+        const f32x4 v4 = *(lds_f4*)(uintptr_t)(lva + (32 * sb + 16 * (q >> 1) + 4 * (q & 1)) * 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) lv[sb][4 * q + e] = v4[e];
+      };
+      // reads due at `slot` (or, for slot 0, everything due at or before it)
+      auto side_reads = [&](auto slot_c) __attribute__((always_inline)) {
+        constexpr int slot = decltype(slot_c)::value;
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int due = use_slot(sb, 2 * q) - 2;
+            if (due == slot || (slot == 0 && due < 0)) load_lv(sb, q);
+          }
+          if (grad) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              const int due = use_slot(sb, 4 * h) - 2;
+              if (due == slot || (slot == 0 && due < 0)) pp[sb][h] = *(lds_i32x4*)(uintptr_t)(pbv + sb * 2048 + h * 1024);
+            }
+          }
+        }
+      };
+      f32x16 S0 = (f32x16){0}, S1 = (f32x16){0};
+      uint32_t W0[8], W1[8];
+      // pair i of a block: P (score wave) or dS (grad wave), rounded and packed
+      auto pair = [&](const f32x16& S, const float* lvb, const i32x4* ppb, int i) __attribute__((always_inline)) -> uint32_t {
+        if (!grad) {
+          return Elem<T>::pack2(fast_exp2(fmaf(S[2 * i], scale, -lvb[2 * i])),
+                                fast_exp2(fmaf(S[2 * i + 1], scale, -lvb[2 * i + 1])));
+        } else {
+          const uint32_t pk = (uint32_t)(i < 4 ? ppb[0][i] : ppb[1][i - 4]);
+          float plo, phi;
+          if (std::is_same<T, __bf16>::value) {
+            plo = __builtin_bit_cast(float, pk << 16);
+            phi = __builtin_bit_cast(float, pk & 0xffff0000u);
+          } else {
+            const f16x2 h2 = __builtin_bit_cast(f16x2, pk);
+            plo = (float)h2[0];
+            phi = (float)h2[1];
+          }
+          return Elem<T>::pack2(plo * (S[2 * i] - lvb[2 * i]), phi * (S[2 * i + 1] - lvb[2 * i + 1]));
+        }
+      };
+      i32x4 f[kPrefetch];
+#pragma unroll
+      for (int st = 0; st < kPrefetch; ++st) f[st] = st < K ? fr.rows(0, 0, st) : fr.rows(0, 1, st - K);
+      __builtin_amdgcn_s_setprio(1);
+      // 1. chain of block 0
+      static_for<0, K>([&](auto st_c) __attribute__((always_inline)) {
+        constexpr int st = decltype(st_c)::value;
+        S0 = Elem<T>::mfma(f[st % kPrefetch], Xf[st], S0);
+        constexpr int nx = st + kPrefetch;
+        f[st % kPrefetch] = nx < K ? fr.rows(0, 0, nx) : fr.rows(0, 1, nx - K);
+        side_reads(ic<st>{});
+        if (st == 1) drip(0);
+        if (st == K / 2 + 1) drip(1);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      // 2. chain of block 1, arithmetic of block 0
+      i32x4 tf[2];
+      tf[0] = fr.tr(0, 0, 0);
+      tf[1] = fr.tr(0, 0, 1);
+      static_for<0, K>([&](auto st_c) __attribute__((always_inline)) {
+        constexpr int st = decltype(st_c)::value;
+        S1 = Elem<T>::mfma(f[(st + K) % kPrefetch], Xf[st], S1);
+        constexpr int nx = st + kPrefetch;
+        if (nx < K) f[(st + K) % kPrefetch] = fr.rows(0, 1, nx);
+        side_reads(ic<K + st>{});
+#pragma unroll
+        for (int i = st * 8 / K; i < (st + 1) * 8 / K; ++i) {
+          W0[i] = pair(S0, lv[0], pp[0], i);
+          asm volatile("" : "+v"(W0[i]));  // computed here, behind this MFMA
+        }
+        if (st == 1) drip(2);
+        if (st == K / 2 + 1) drip(3);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      if (!grad) {
+        *(lds_i32x4*)(uintptr_t)(pbv) = (i32x4){(int)W0[0], (int)W0[1], (int)W0[2], (int)W0[3]};
+        *(lds_i32x4*)(uintptr_t)(pbv + 1024) = (i32x4){(int)W0[4], (int)W0[5], (int)W0[6], (int)W0[7]};
+      }
+      __builtin_amdgcn_s_setprio(3);
+      // 3. accumulating product of block 0, arithmetic of block 1
+      static_for<0, NACC>([&](auto i_c) __attribute__((always_inline)) {
+        constexpr int i = decltype(i_c)::value;
+        constexpr int kk = i / G::NDB, db = i % G::NDB;
+        const i32x4 wf = {(int)W0[4 * kk], (int)W0[4 * kk + 1], (int)W0[4 * kk + 2], (int)W0[4 * kk + 3]};
+        acc[db] = Elem<T>::mfma(tf[i & 1], wf, acc[db]);
+        constexpr int nx = i + 2;
+        tf[i & 1] = nx < NACC ? fr.tr(0, nx / G::NDB, nx % G::NDB) : fr.tr(0, 2 + (nx - NACC) / G::NDB, (nx - NACC) % G::NDB);
+        side_reads(ic<2 * K + i>{});
+#pragma unroll
+        for (int j = i * 8 / NACC; j < (i + 1) * 8 / NACC; ++j) {
+          W1[j] = pair(S1, lv[1], pp[1], j);
+          asm volatile("" : "+v"(W1[j]));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      if (!grad) {
+        *(lds_i32x4*)(uintptr_t)(pbv + 2048) = (i32x4){(int)W1[0], (int)W1[1], (int)W1[2], (int)W1[3]};
+        *(lds_i32x4*)(uintptr_t)(pbv + 2048 + 1024) = (i32x4){(int)W1[4], (int)W1[5], (int)W1[6], (int)W1[7]};
+      }
+      // 4. accumulating product of block 1
+#pragma unroll
+      for (int i = 0; i < NACC; ++i) {
+        const int kk = i / G::NDB, db = i % G::NDB;
+        const i32x4 wf = {(int)W1[4 * kk], (int)W1[4 * kk + 1], (int)W1[4 * kk + 2], (int)W1[4 * kk + 3]};
+        acc[db] = Elem<T>::mfma(tf[i & 1], wf, acc[db]);
+        if (i + 2 < NACC) tf[i & 1] = fr.tr(0, 2 + (i + 2) / G::NDB, (i + 2) % G::NDB);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  // Tiles on the diagonal or at the sequence end: block by block, with masks.
+  auto compute_slow = [&](auto role_c) __attribute__((always_inline)) {
+    constexpr bool grad = decltype(role_c)::value != 0;
+    const int s0 = cmp_s0;
+    drip_all();
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
       const int sblk = s0 + 32 * sb;
@@ -611,35 +831,29 @@ __device__ __forceinline__ void bwd_dkdv_item(const BwdParams& p, const int bid,
       for (int g2 = 0; g2 < 2; ++g2)
 #pragma unroll
         for (int q4 = 0; q4 < 2; ++q4) {
-          const uint32_t a = lds0 + LV + (grad ? 256u : 0u) + (32 * sb + 16 * g2 + 8 * fr.lh + 4 * q4) * 4;
-          const f32x4 lv = *(lds_f4*)(uintptr_t)a;
+          const f32x4 v4 = *(lds_f4*)(uintptr_t)(lva + (32 * sb + 16 * g2 + 4 * q4) * 4);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) vec_r[8 * g2 + 4 * q4 + e] = lv[e];
+          for (int e = 0; e < 4; ++e) vec_r[8 * g2 + 4 * q4 + e] = v4[e];
         }
       // first product: rows of Q (score) / dO (grad) against the resident operand
-      constexpr uint32_t TR = grad ? T1 : T0;   // tile read as row fragments
-      constexpr uint32_t TT = grad ? T0 : T1;   // tile read transposed for the accumulating product
       f32x16 S = (f32x16){0};
       i32x4 f[kPrefetch];
 #pragma unroll
-      for (int st = 0; st < kPrefetch; ++st) f[st] = fr.rows(TR, sb, st);
-      // Issue priority: low during the serial chain and the arithmetic behind
-      // it, high while the wave feeds its accumulators (NDB independent chains),
-      // so that the two waves of a SIMD fall out of step.
+      for (int st = 0; st < kPrefetch; ++st) f[st] = fr.rows(0, sb, st);
       __builtin_amdgcn_s_setprio(1);
 #pragma unroll
       for (int st = 0; st < G::KSTEPS; ++st) {
         S = Elem<T>::mfma(f[st % kPrefetch], Xf[st], S);
-        if (st + kPrefetch < G::KSTEPS) f[st % kPrefetch] = fr.rows(TR, sb, st + kPrefetch);
+        if (st + kPrefetch < G::KSTEPS) f[st % kPrefetch] = fr.rows(0, sb, st + kPrefetch);
         __builtin_amdgcn_sched_barrier(0);
       }
       i32x4 tf[2];
-      tf[0] = fr.tr(TT, 2 * sb, 0);
-      tf[1] = fr.tr(TT, 2 * sb, 1);
+      tf[0] = fr.tr(0, 2 * sb, 0);
+      tf[1] = fr.tr(0, 2 * sb, 1);
       uint32_t W[8];
       if (!grad) {
-        // rare: rows / columns that do not exist or lie above the diagonal give P = 0
-        bool need_mask = sblk + 32 > len || r0w + 32 > len;
+        // rows / columns that do not exist or lie above the diagonal give P = 0
+        bool need_mask = sblk + 32 > len || !rows_full;
         if (causal) need_mask = need_mask || sblk < r0w + 31;
         if (need_mask) {
 #pragma unroll
@@ -654,11 +868,11 @@ __device__ __forceinline__ void bwd_dkdv_item(const BwdParams& p, const int bid,
           W[i] = Elem<T>::pack2(fast_exp2(fmaf(S[2 * i], scale, -vec_r[2 * i])),
                                 fast_exp2(fmaf(S[2 * i + 1], scale, -vec_r[2 * i + 1])));
         // P for the grad wave of this group (it reads it in the next tile step)
-        *(lds_i32x4*)(uintptr_t)(pb + sb * 2048) = (i32x4){(int)W[0], (int)W[1], (int)W[2], (int)W[3]};
-        *(lds_i32x4*)(uintptr_t)(pb + sb * 2048 + 1024) = (i32x4){(int)W[4], (int)W[5], (int)W[6], (int)W[7]};
+        *(lds_i32x4*)(uintptr_t)(pbv + sb * 2048) = (i32x4){(int)W[0], (int)W[1], (int)W[2], (int)W[3]};
+        *(lds_i32x4*)(uintptr_t)(pbv + sb * 2048 + 1024) = (i32x4){(int)W[4], (int)W[5], (int)W[6], (int)W[7]};
       } else {
-        const i32x4 p0 = *(lds_i32x4*)(uintptr_t)(pb + sb * 2048);
-        const i32x4 p1 = *(lds_i32x4*)(uintptr_t)(pb + sb * 2048 + 1024);
+        const i32x4 p0 = *(lds_i32x4*)(uintptr_t)(pbv + sb * 2048);
+        const i32x4 p1 = *(lds_i32x4*)(uintptr_t)(pbv + sb * 2048 + 1024);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           const uint32_t pk = (uint32_t)(i < 4 ? p0[i] : p1[i - 4]);
@@ -682,7 +896,7 @@ __device__ __forceinline__ void bwd_dkdv_item(const BwdParams& p, const int bid,
         const int kk = i / G::NDB, db = i % G::NDB;
         const i32x4 wf = {(int)W[4 * kk], (int)W[4 * kk + 1], (int)W[4 * kk + 2], (int)W[4 * kk + 3]};
         acc[db] = Elem<T>::mfma(tf[i & 1], wf, acc[db]);
-        if (i + 2 < NACC) tf[i & 1] = fr.tr(TT, 2 * sb + (i + 2) / G::NDB, (i + 2) % G::NDB);
+        if (i + 2 < NACC) tf[i & 1] = fr.tr(0, 2 * sb + (i + 2) / G::NDB, (i + 2) % G::NDB);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -690,34 +904,63 @@ __device__ __forceinline__ void bwd_dkdv_item(const BwdParams& p, const int bid,
 
   // step i: the score waves work on tile i, the grad waves on tile i - 1, and
   // tile i + 1 is on its way into the stage that tile i - 2 has left
-  if (n_stream > 0) issue();
+  if (n_stream > 0) {
+    request();
+    drip_all();
+    advance();
+  }
   __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
   __syncthreads();
-  auto step = [&](auto role_c, auto stage_c, int i) __attribute__((always_inline)) {
-    if (i + 1 < n_stream) issue();
-    if (decltype(role_c)::value ? i >= 1 : i < n_stream) compute(role_c, stage_c);
+  auto sync_step = [&]() __attribute__((always_inline)) {
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __syncthreads();
   };
-  if (!grad) {
-    for (int i = 0; i <= n_stream; i += NS) {
-      step(ic<0>{}, ic<0>{}, i);
-      if (i + 1 > n_stream) break;
-      step(ic<0>{}, ic<1>{}, i + 1);
-      if (i + 2 > n_stream) break;
-      step(ic<0>{}, ic<2>{}, i + 2);
+  // Tiles of a head that need masks: the first ones of a causal item (keys of
+  // this group against queries at or before them) and a last, partial one.
+  int n_pre = causal ? (32 * pr + 31 + TN - 1) / TN : 0;
+  int n_post = (len % TN) != 0 ? 1 : 0;
+  if (!rows_full) n_pre = nj;
+  n_pre = min(n_pre, nj);
+  n_post = min(n_post, nj - n_pre);
+  int req_left = n_stream - 1;  // requests still to make (the first one is out)
+  // Each loop below holds ONE kind of step: with the masked path and the
+  // pipelined path in one loop body the accumulators were copied between two
+  // register sets on every trip.
+  auto run = [&](auto role_c) __attribute__((always_inline)) {
+    constexpr bool gr = decltype(role_c)::value != 0;
+    auto step = [&](auto fast_c) __attribute__((always_inline)) {
+      const bool more = req_left > 0;
+      if (more) request();
+      if (decltype(fast_c)::value)
+        compute_fast(role_c);
+      else
+        compute_slow(role_c);
+      rotate();
+      if (more) advance();
+      --req_left;
+      sync_step();
+    };
+    if (gr) {  // step 0: nothing to work on yet
+      if (req_left > 0) {
+        request();
+        drip_all();
+        advance();
+      }
+      --req_left;
+      sync_step();
     }
-  } else {
-    step(ic<1>{}, ic<0>{}, 0);  // nothing to work on yet
-    for (int i = 1; i <= n_stream; i += NS) {
-      step(ic<1>{}, ic<0>{}, i);
-      if (i + 1 > n_stream) break;
-      step(ic<1>{}, ic<1>{}, i + 1);
-      if (i + 2 > n_stream) break;
-      step(ic<1>{}, ic<2>{}, i + 2);
+    for (int g = 0; g < gqa; ++g) {
+      for (int jj = 0; jj < n_pre; ++jj) step(ic<0>{});
+      for (int jj = n_pre; jj < nj - n_post; ++jj) step(ic<1>{});
+      for (int jj = nj - n_post; jj < nj; ++jj) step(ic<0>{});
     }
-  }
+    if (!gr) sync_step();  // the grad waves' last tile
+  };
+  if (!grad)
+    run(ic<0>{});
+  else
+    run(ic<1>{});
 
   // ---- epilogue: dV from the score waves, dK from the grad waves
   const float oscale = grad ? p.scale_nat : 1.f;
