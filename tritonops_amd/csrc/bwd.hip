@@ -545,39 +545,46 @@ __device__ __forceinline__ void bwd_dkdv_item(const BwdParams& p, const int bid,
   const uint64_t wrap0 = uniform64((uint64_t)(p.q_sh * 2 - (int64_t)(nj - 1) * TN * pitch0));
   const uint64_t wrap1 = uniform64((uint64_t)(p.do_sh * 2 - (int64_t)(nj - 1) * TN * pitch1));
   const uint64_t wrapl = uniform64((uint64_t)((wave == 0 ? p.lse_sh * 4 : p.dl_sh * 4) - (int64_t)(nj - 1) * TN * pitchl));
-  uint32_t off0[IPW], off1[IPW];
-  uint64_t lane_mask[IPW];
-#pragma unroll
-  for (int t = 0; t < IPW; ++t) {
-    const int r = RPI * (wave + NW * t) + drow;
+  // The four score wavefronts send the loads (the grad wavefronts carry more
+  // arithmetic per tile): wave pr sends slabs pr, pr + 4, pr + 8, pr + 12 of
+  // the Q tile and of the dO tile (1 KiB = four rows each).  The swizzle of a
+  // lane's chunk depends on the slab only through slab % 4, so one lane offset
+  // per tensor serves all four slabs; the slab moves the scalar base.
+  constexpr int kSlabs = TN / RPI / NP;      // slabs per tensor, tile and score wave
+  constexpr int kDrips = 2 * kSlabs;
+  static_assert(kDrips == 8, "compute_fast() places eight loads");
+  uint32_t off0, off1;
+  uint64_t lane_mask;
+  {
+    const int r = RPI * pr + drow;
     const int c = dslot ^ F::swz(r);
-    off0[t] = (uint32_t)r * (uint32_t)pitch0 + c * 16;
-    off1[t] = (uint32_t)r * (uint32_t)pitch1 + c * 16;
-    lane_mask[t] = __builtin_amdgcn_ballot_w64(G::NCH == 16 || c < G::NCH);
+    off0 = (uint32_t)r * (uint32_t)pitch0 + c * 16;
+    off1 = (uint32_t)r * (uint32_t)pitch1 + c * 16;
+    lane_mask = __builtin_amdgcn_ballot_w64(G::NCH == 16 || c < G::NCH);
   }
+  const uint64_t slab0 = uniform64((uint64_t)(NP * RPI * pitch0)), slab1 = uniform64((uint64_t)(NP * RPI * pitch1));
   const uint32_t lv_off = (uint32_t)lane * (uint32_t)pitchl;
   const uint64_t lv_mask = wave < 2 ? ~0ull : 0ull;
-  constexpr int kDrips = 2 * IPW;
-  static_assert(kDrips == 4, "compute() places four loads");
   int iss_left = nj;        // tiles of the current head still to request
   int iss_s0 = j0 * TN;     // first row of the next request
   int iss_st = 0;           // its stage
   uint32_t iss_base = lds0; // and the stage's LDS address
-  uint64_t drip_on = 0;     // all ones while the loads of a request are still to be sent by compute()
+  uint64_t drip_on = 0;     // all ones while the loads of a request are still to be sent by compute_fast()
   // request(): a tile that reaches past the sequence end is loaded at once,
   // row by row with clamped row numbers (masked later); a full tile only arms
-  // drip(), and compute() sends the four loads between its MFMAs: eight
-  // wavefronts that send their loads together right after the barrier stand
-  // in the memory pipeline's queue before any of them starts its arithmetic.
+  // drip(), and compute_fast() sends the loads between its MFMAs: wavefronts
+  // that send their loads together right after the barrier stand in the
+  // memory pipeline's queue before any of them starts its arithmetic.
   auto request = [&]() __attribute__((always_inline)) {
     if (iss_s0 + TN <= len) {
       drip_on = ~0ull;
     } else {
       drip_on = 0;
+      if (grad) return;
       const int last = len - 1 - iss_s0;  // >= 0
 #pragma unroll
-      for (int t = 0; t < IPW; ++t) {
-        const int inst = wave + NW * t;
+      for (int t = 0; t < kSlabs; ++t) {
+        const int inst = pr + NP * t;
         const int r = RPI * inst + drow;
         const int c = dslot ^ F::swz(r);
         const int64_t rr = min(r, last);
@@ -597,16 +604,18 @@ __device__ __forceinline__ void bwd_dkdv_item(const BwdParams& p, const int bid,
       }
     }
   };
+  // load k of a request (score waves): k & 1 = tensor, k >> 1 = slab
   auto drip = [&](int k) __attribute__((always_inline)) {
     const int t = k >> 1;
-    const int inst = wave + NW * t;
+    const int inst = pr + NP * t;
     if (k & 1)
-      dma_masked(drip_on & lane_mask[t], a1, off1[t], iss_base + TILEB + inst * 1024, ic<1>{});
+      dma_masked(drip_on & lane_mask, a1 + t * slab1, off1, iss_base + TILEB + inst * 1024, ic<1>{});
     else
-      dma_masked(drip_on & lane_mask[t], a0, off0[t], iss_base + inst * 1024, ic<1>{});
+      dma_masked(drip_on & lane_mask, a0 + t * slab0, off0, iss_base + inst * 1024, ic<1>{});
     if (k == 0) dma_masked(drip_on & lv_mask, al, lv_off, iss_base + 2 * TILEB + (wave == 0 ? 0 : 256), ic<0>{});
   };
   auto drip_all = [&]() __attribute__((always_inline)) {
+    if (grad) return;
 #pragma unroll
     for (int k = 0; k < kDrips; ++k) drip(k);
   };
@@ -695,6 +704,8 @@ __device__ __forceinline__ void bwd_dkdv_item(const BwdParams& p, const int bid,
       // read) and the packed P a pair needs are read two slots earlier, so
       // that only a few of them are live at a time (registers).
       constexpr int K = G::KSTEPS;
+      // slice of a chain phase behind which the n-th of its four loads goes
+      auto drip_slice = [](int n) constexpr { return K == 8 ? 2 * n + 1 : K == 6 ? n + 1 + (n >= 2) : n; };
       auto slice_of = [](int i, int n) constexpr { int st = 0; while ((st + 1) * 8 / n <= i) ++st; return st; };
       auto use_slot = [&](int sb, int i) constexpr { return sb == 0 ? K + slice_of(i, K) : 2 * K + slice_of(i, NACC); };
       float lv[2][16];
@@ -755,8 +766,10 @@ __device__ __forceinline__ void bwd_dkdv_item(const BwdParams& p, const int bid,
         constexpr int nx = st + kPrefetch;
         f[st % kPrefetch] = nx < K ? fr.rows(0, 0, nx) : fr.rows(0, 1, nx - K);
         side_reads(ic<st>{});
-        if (st == 1) drip(0);
-        if (st == K / 2 + 1) drip(1);
+        if (!grad)
+          static_for<0, 4>([&](auto n_c) __attribute__((always_inline)) {
+            if (st == drip_slice(decltype(n_c)::value)) drip(decltype(n_c)::value);
+          });
         __builtin_amdgcn_sched_barrier(0);
       });
       // 2. chain of block 1, arithmetic of block 0
@@ -774,8 +787,10 @@ __device__ __forceinline__ void bwd_dkdv_item(const BwdParams& p, const int bid,
           W0[i] = pair(S0, lv[0], pp[0], i);
           asm volatile("" : "+v"(W0[i]));  // computed here, behind this MFMA
         }
-        if (st == 1) drip(2);
-        if (st == K / 2 + 1) drip(3);
+        if (!grad)
+          static_for<0, 4>([&](auto n_c) __attribute__((always_inline)) {
+            if (st == drip_slice(decltype(n_c)::value)) drip(4 + decltype(n_c)::value);
+          });
         __builtin_amdgcn_sched_barrier(0);
       });
       if (!grad) {
