@@ -146,6 +146,52 @@ struct TileDma {
                  : "memory");
   }
 
+  // A load of the lanes in `mask`, for straight-line code between MFMAs
+  // (all 64 lanes are active and control flow is wave-uniform where it is
+  // used, so exec is restored to all ones; a branch around the load would end
+  // the basic block and the pinned instruction order with it).
+  static __device__ __forceinline__ void dma16m(uint64_t mask, uint64_t base, uint32_t off, uint32_t slab) {
+    asm volatile("s_mov_b32 m0, %3\n\ts_mov_b64 exec, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, -1"
+                 :
+                 : "s"(mask), "v"(off), "s"(base), "s"(slab)
+                 : "memory");
+  }
+
+  // Loads of one whole tile, sent one at a time: arm() fixes the tile
+  // (wave-uniform bases), one(k) sends load k of 2*IPW (K and V alternate).
+  struct Drip {
+    uint64_t on;  // all ones when armed, 0: the loads are no-ops
+    uint64_t kt, vt;
+    uint32_t sK, sV;
+  };
+  template <int ST>
+  __device__ __forceinline__ Drip arm(const KvSrc<T>& s, int k0, bool on) const {
+    Drip d;
+    const uint32_t k0u = (uint32_t)__builtin_amdgcn_readfirstlane(k0);
+    d.on = uniform64(on ? ~0ull : 0ull);
+    d.kt = uniform64(s.k_base + (uint64_t)k0u * k_pitch);
+    d.vt = uniform64(s.v_base + (uint64_t)k0u * v_pitch);
+    d.sK = lds0 + ST * TILEB;
+    d.sV = lds0 + VBASE + ST * TILEB;
+    return d;
+  }
+  __device__ __forceinline__ void one(const Drip& d, int k) const {
+    const int t = k >> 1;
+    const int inst = wave + NW * t;
+    uint64_t mask = d.on;
+    if (D == 96) {
+      int ln = lane;
+      const int drow = ln / F::SLOTS, dslot = ln % F::SLOTS;
+      const int r = RPI * inst + drow;
+      const int c = dslot ^ ((k & 1) ? F::swz_v(r) : F::swz_k(r));
+      mask = uniform64(mask & __builtin_amdgcn_ballot_w64(c < G::NCH));
+    }
+    if (k & 1)
+      dma16m(mask, d.vt, voff[t], d.sV + inst * 1024);
+    else
+      dma16m(mask, d.kt, koff[t], d.sK + inst * 1024);
+  }
+
   __device__ __forceinline__ void init(const PrefillParams& p, int lane_, int wave_) {
     lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem);
     wave = wave_;
@@ -304,9 +350,17 @@ sparse_kernel(const PrefillParams p) {
       col_cur = col_nxt;
       col_nxt = load_cols(col_chunk + 1);
     }
-    // refill the stage that was read in the previous iteration
+    // refill the stage that was read in the previous iteration: a tile that
+    // reaches past the sequence end at once (clamped rows), a whole tile one
+    // load at a time behind the MFMAs of the score chain below.  (Sent in
+    // one go right after the barrier, the eight loads of a wave queue up in
+    // the memory pipeline behind the other waves' and the wave reaches its
+    // arithmetic hundreds of cycles later.)
     const bool refill = it + NS - 1 < n_tiles;
-    if (refill) dma.template tile<(ST + NS - 1) % NS>(kv, tile_k0(it + NS - 1));
+    const int k0r = refill ? tile_k0(it + NS - 1) : 0;
+    const bool whole = k0r + TN <= len;
+    if (refill && !whole) dma.template tile<(ST + NS - 1) % NS>(kv, k0r);
+    const typename DMA::Drip drip = dma.template arm<(ST + NS - 1) % NS>(kv, k0r, refill && whole);
 
     const int k0 = tile_k0(it);
     // whole tile above the diagonal for this wave: nothing to add
@@ -323,7 +377,30 @@ sparse_kernel(const PrefillParams p) {
         return ok;
       };
       // V addresses carry VBASE inside the lane offsets (see fr.init)
-      compute_tile<T, D, TN / 32>((uint32_t)(ST * TILEB), (uint32_t)(ST * TILEB), fr, Qf, O, m, l, p.scale, need_mask, allowed);
+      static_assert(TN == 32, "one 32-key block per tile");
+      constexpr uint32_t sK = ST * TILEB, sV = ST * TILEB;
+      f32x16 S[1];
+      uint32_t P[1][8];
+      {
+        constexpr int kPrefetch = 4;
+        i32x4 kf[kPrefetch];
+#pragma unroll
+        for (int c = 0; c < kPrefetch; ++c) kf[c] = fr.load_k(sK, 0, c);
+        S[0] = (f32x16){0};
+#pragma unroll
+        for (int c = 0; c < G::KSTEPS; ++c) {
+          S[0] = Elem<T>::mfma(kf[c % kPrefetch], Qf[c], S[0]);
+          if (c + kPrefetch < G::KSTEPS) kf[c % kPrefetch] = fr.load_k(sK, 0, c + kPrefetch);
+#pragma unroll
+          for (int k = c * 2 * IPW / G::KSTEPS; k < (c + 1) * 2 * IPW / G::KSTEPS; ++k) dma.one(drip, k);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      softmax_tile<T, D, 1>(S, fr.lh, O, m, l, p.scale, need_mask, allowed, P);
+      pv_accumulate<T, D, 1>(sV, fr, P, O);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 2 * IPW; ++k) dma.one(drip, k);
     }
     // The next tile must have landed and everyone must be done with this one.
     // This wave's loads complete in order, so it is enough that at most the
