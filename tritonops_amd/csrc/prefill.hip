@@ -396,8 +396,58 @@ sparse_kernel(const PrefillParams p) {
           __builtin_amdgcn_sched_barrier(0);
         }
       }
-      softmax_tile<T, D, 1>(S, fr.lh, O, m, l, p.scale, need_mask, allowed, P);
-      pv_accumulate<T, D, 1>(sV, fr, P, O);
+      // Online softmax as in softmax_tile(), with the second half of the
+      // exponentials behind the first MFMAs of O^T += V^T P^T (those need the
+      // probabilities of the lane's first eight keys only) and the V
+      // fragments read two MFMAs ahead.
+      i32x4 vf[2];
+      vf[0] = fr.load_v(sV, 0, 0);
+      vf[1] = fr.load_v(sV, 0, 1 % G::NDB);
+      if (need_mask) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = 16 * (r >> 3) + 8 * fr.lh + (r & 7);
+          if (!allowed(key)) S[0][r] = -INFINITY;
+        }
+      }
+      float mx = S[0][0];
+#pragma unroll
+      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, S[0][r]);
+      mx = max_with_other_half(mx);
+      const float m_new = fmaxf(m, mx * p.scale);
+      if (__builtin_amdgcn_ballot_w64(m_new > m + kRescaleSlack) != 0) {
+        const float alpha = fast_exp2(m - ((m_new == -INFINITY) ? 0.f : m_new));
+        l *= alpha;
+#pragma unroll
+        for (int db = 0; db < G::NDB; ++db) O[db] *= alpha;
+        m = m_new;
+      }
+      const float m_use = (m == -INFINITY) ? 0.f : m;
+      const float sc = p.scale;
+      float rs = 0.f;
+      auto expo = [&](int i) __attribute__((always_inline)) {
+        const float p0 = fast_exp2(fmaf(S[0][2 * i], sc, -m_use));
+        const float p1 = fast_exp2(fmaf(S[0][2 * i + 1], sc, -m_use));
+        rs += p0 + p1;
+        P[0][i] = Elem<T>::pack2(p0, p1);
+        asm volatile("" : "+v"(P[0][i]));
+      };
+#pragma unroll
+      for (int i = 0; i < 4; ++i) expo(i);
+      __builtin_amdgcn_sched_barrier(0);
+      constexpr int NACC = 2 * G::NDB;
+#pragma unroll
+      for (int i = 0; i < NACC; ++i) {
+        const int kk = i / G::NDB, db = i % G::NDB;
+        const i32x4 pf = {(int)P[0][4 * kk], (int)P[0][4 * kk + 1], (int)P[0][4 * kk + 2], (int)P[0][4 * kk + 3]};
+        O[db] = Elem<T>::mfma(vf[i & 1], pf, O[db]);
+        if (i + 2 < NACC) vf[i & 1] = fr.load_v(sV, (i + 2) / G::NDB, (i + 2) % G::NDB);
+#pragma unroll
+        for (int j = 4 + i * 4 / G::NDB; j < 4 + (i + 1) * 4 / G::NDB; ++j)
+          if (i < G::NDB) expo(j);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      l += rs;
     } else {
 #pragma unroll
       for (int k = 0; k < 2 * IPW; ++k) dma.one(drip, k);
