@@ -193,117 +193,158 @@ __device__ __forceinline__ void bwd_dq_item(const BwdParams& p, const int bid) {
 
   // ---- direct-to-LDS loads (inline assembly: see the note in prefill.hip)
   const int drow = lane / F::SLOTS, dslot = lane % F::SLOTS;
-  auto dma16 = [&](const char* g, uint32_t slab_u) __attribute__((always_inline)) {
-    const uint32_t slab = (uint32_t)__builtin_amdgcn_readfirstlane(slab_u);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(slab) : "memory");
-  };
-  // the same with the address as "uniform 64-bit base + 32-bit lane offset":
-  // no vector arithmetic per load
-  auto dma16s = [&](uint64_t base, uint32_t off, uint32_t slab_u) __attribute__((always_inline)) {
-    const uint32_t slab = (uint32_t)__builtin_amdgcn_readfirstlane(slab_u);
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"(base), "s"(slab) : "memory");
-  };
   auto uniform64 = [](uint64_t x) __attribute__((always_inline)) -> uint64_t {
     const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)x);
     const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(x >> 32));
     return ((uint64_t)hi << 32) | lo;
   };
+  // a load of the lanes in `mask` in straight-line code (all lanes are active
+  // and control flow is wave-uniform here: exec is restored to all ones)
+  auto dma_masked = [&](uint64_t mask, uint64_t base, uint32_t off, uint32_t slab) __attribute__((always_inline)) {
+    asm volatile("s_mov_b32 m0, %3\n\ts_mov_b64 exec, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, -1"
+                 : : "s"(mask), "v"(off), "s"(base), "s"(slab) : "memory");
+  };
   // Streamed tensors: K feeds the first product and, transposed, the last; V
-  // the second.  Their row pitches and this lane's offsets inside a tile are
-  // fixed for the item.
+  // the second.  Wave w sends slabs w and w + 8 (1 KiB = four rows) of either
+  // tile; the swizzle of a lane's chunk depends on the slab only through
+  // slab % 4, so one lane offset per tensor serves both and the slab moves the
+  // scalar base.  The tile addresses are running, wave-uniform values.
   const int64_t pitch0 = p.k_ss * 2, pitch1 = p.v_ss * 2;
   const int hs = hr / gqa;
   const char* h0 = reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.k) + bsel * p.k_sb + start * p.k_ss + hs * p.k_sh);
   const char* h1 = reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.v) + bsel * p.v_sb + start * p.v_ss + hs * p.v_sh);
-  uint32_t off0[IPW], off1[IPW];
-#pragma unroll
-  for (int t = 0; t < IPW; ++t) {
-    const int r = RPI * (wave + NW * t) + drow;
+  uint64_t a0 = uniform64((uint64_t)(uintptr_t)h0), a1 = uniform64((uint64_t)(uintptr_t)h1);
+  const uint64_t step0 = uniform64((uint64_t)(TN * pitch0)), step1 = uniform64((uint64_t)(TN * pitch1));
+  const uint64_t slab0 = uniform64((uint64_t)(NW * RPI * pitch0)), slab1 = uniform64((uint64_t)(NW * RPI * pitch1));
+  uint32_t off0, off1;
+  uint64_t lane_mask;
+  {
+    const int r = RPI * wave + drow;
     const int c = dslot ^ F::swz(r);
-    off0[t] = (uint32_t)r * (uint32_t)pitch0 + c * 16;
-    off1[t] = (uint32_t)r * (uint32_t)pitch1 + c * 16;
+    off0 = (uint32_t)r * (uint32_t)pitch0 + c * 16;
+    off1 = (uint32_t)r * (uint32_t)pitch1 + c * 16;
+    lane_mask = __builtin_amdgcn_ballot_w64(G::NCH == 16 || c < G::NCH);
   }
-  // key tile u into stage ST
-  auto issue = [&](int u, auto stage_c) __attribute__((always_inline)) {
-    constexpr int ST = decltype(stage_c)::value;
-    const int s0 = u * TN;
-    const uint32_t base = lds0 + ST * STAGEB;
-    if (s0 + TN <= len) {
-      const uint64_t a0 = uniform64((uint64_t)(uintptr_t)(h0 + s0 * pitch0));
-      const uint64_t a1 = uniform64((uint64_t)(uintptr_t)(h1 + s0 * pitch1));
-#pragma unroll
-      for (int t = 0; t < IPW; ++t) {
-        const int inst = wave + NW * t;
-        const int c = dslot ^ F::swz(RPI * inst + drow);
-        if (G::NCH == 16 || c < G::NCH) {
-          dma16s(a0, off0[t], base + inst * 1024);
-          dma16s(a1, off1[t], base + TILEB + inst * 1024);
-        }
-      }
+  static_assert(IPT == 4, "compute_fast() places four loads");
+  int iss_s0 = 0;            // first row of the next request
+  int iss_st = 0;            // its stage
+  uint32_t iss_base = lds0;  // and the stage's LDS address
+  uint64_t drip_on = 0;      // all ones while the loads of a request are still to be sent by a compute step
+  // request(): a tile that reaches past the sequence end is loaded at once,
+  // row by row with clamped row numbers (masked later); a whole tile only arms
+  // drip(), and the compute step sends the four loads between its MFMAs.
+  auto request = [&]() __attribute__((always_inline)) {
+    if (iss_s0 + TN <= len) {
+      drip_on = ~0ull;
     } else {
+      drip_on = 0;
+      const int last = len - 1 - iss_s0;  // >= 0
 #pragma unroll
       for (int t = 0; t < IPW; ++t) {
         const int inst = wave + NW * t;
         const int r = RPI * inst + drow;
         const int c = dslot ^ F::swz(r);
-        const int64_t rr = min(s0 + r, len - 1);  // rows past the end re-read the last row (masked later)
+        const int64_t rr = min(r, last);
+        const uint32_t slab = (uint32_t)__builtin_amdgcn_readfirstlane(iss_base + inst * 1024);
         if (G::NCH == 16 || c < G::NCH) {
-          dma16(h0 + rr * pitch0 + c * 16, base + inst * 1024);
-          dma16(h1 + rr * pitch1 + c * 16, base + TILEB + inst * 1024);
+          asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                       : : "v"((const char*)a0 + rr * pitch0 + c * 16), "s"(slab) : "memory");
+          asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                       : : "v"((const char*)a1 + rr * pitch1 + c * 16), "s"(slab + TILEB) : "memory");
         }
       }
     }
+  };
+  // load k of a request: k & 1 = tensor, k >> 1 = slab
+  auto drip = [&](int k) __attribute__((always_inline)) {
+    const int t = k >> 1;
+    const int inst = wave + NW * t;
+    if (k & 1)
+      dma_masked(drip_on & lane_mask, a1 + t * slab1, off1, iss_base + TILEB + inst * 1024);
+    else
+      dma_masked(drip_on & lane_mask, a0 + t * slab0, off0, iss_base + inst * 1024);
+  };
+  auto drip_all = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int k = 0; k < IPT; ++k) drip(k);
+  };
+  auto advance = [&]() __attribute__((always_inline)) {
+    drip_on = 0;
+    iss_s0 += TN;
+    a0 += step0;
+    a1 += step1;
+    const bool last_st = iss_st == NS - 1;
+    iss_st = last_st ? 0 : iss_st + 1;
+    iss_base = last_st ? lds0 : iss_base + STAGEB;
   };
 
   const float scale = p.scale;
   const int causal = p.causal;
 
-  auto compute = [&](int u, auto stage_c) __attribute__((always_inline)) {
-    constexpr int ST = decltype(stage_c)::value;
-    constexpr uint32_t T0 = ST * STAGEB, T1 = ST * STAGEB + TILEB;
-    const int s0 = u * TN;
-    constexpr int kPrefetch = 4;
-    i32x4 f[kPrefetch];   // row fragments of the first product, read ahead
-    bool f_ready = false; // block 0 has already fetched the first fragments of block 1
+  // ---- this wave's view of the tile it works on: LDS addresses that move
+  // from stage to stage (one add per address register and step; every read is
+  // then "register + immediate": absolute stage offsets exceed the 16-bit
+  // immediate of an LDS instruction)
+  int cmp_st = 0;
+  auto rotate = [&]() __attribute__((always_inline)) {
+    const bool last_st = cmp_st == NS - 1;
+    const int d = last_st ? -(NS - 1) * STAGEB : STAGEB;
+    cmp_st = last_st ? 0 : cmp_st + 1;
 #pragma unroll
-    for (int sb = 0; sb < 2; ++sb) {
-      const int sblk = s0 + 32 * sb;
-      if (sblk >= len) continue;
-      if (causal && sblk > r0w + 31) continue;  // keys past this wave's last query
-      // register r of this lane is streamed row  sblk + 16*(r/8) + 8*lh + r%8
-      // The block as one pinned instruction stream (sched_barrier(0) after every
-      // slice): the S chain; the dP chain with the exponentials of S behind its
-      // MFMAs; the first half of dS; the last product with the second half of
-      // dS behind its first MFMAs.  Row fragments are read four steps ahead,
-      // transposed fragments two.
-      constexpr int NSTEP = 2 * G::KSTEPS;
-      constexpr uint32_t TT = T0;  // tile whose transpose is the A operand of the last product
-      f32x16 S = (f32x16){0}, dP = (f32x16){0};
-      auto frag = [&](int st) __attribute__((always_inline)) -> i32x4 {
-        return st < G::KSTEPS ? fr.rows(T0, sb, st) : fr.rows(T1, sb, st - G::KSTEPS);
-      };
-      auto prob = [&](int r) __attribute__((always_inline)) {   // S[r] <- P[r]
-        S[r] = fast_exp2(fmaf(S[r], scale, -lse_l));
-      };
-      auto dsv = [&](int r) __attribute__((always_inline)) -> float {
-        return S[r] * (dP[r] - delta_l);
-      };
-      if (!f_ready) {
+    for (int c = 0; c < G::KSTEPS; ++c) fr.r_a[c] += d;
 #pragma unroll
-        for (int st = 0; st < kPrefetch; ++st) f[st] = frag(st);
-      }
-      // Issue priority: highest while the wave feeds the accumulators (the last
-      // product, 2*NDB MFMAs over NDB independent chains), low during the two
-      // serial chains S and dP; the two waves of a SIMD then fall out of step
-      // instead of competing with the same kind of work (measured 3 %).
-      __builtin_amdgcn_s_setprio(1);
+    for (int db = 0; db < G::NDB; ++db) {
+      fr.t_a[db][0] += d;
+      fr.t_a[db][1] += d;
+    }
+  };
+
+  constexpr int kPrefetch = 4;
+  constexpr int K = G::KSTEPS;
+  // slice of block 0's S chain behind which the n-th of a tile's four loads goes
+  auto drip_slice = [](int n) constexpr { return K == 8 ? 2 * n + 1 : K == 6 ? n + 1 + (n >= 2) : n; };
+  i32x4 f[kPrefetch];   // row fragments of the first two products, read ahead
+  // One 32-row block of the streamed tile as one pinned instruction stream
+  // (sched_barrier(0) after every slice): the S chain; the dP chain with the
+  // exponentials of S behind its MFMAs; the first half of dS; the last product
+  // with the second half of dS behind its first MFMAs.  Row fragments are read
+  // four steps ahead, transposed fragments two.  Register r of this lane is
+  // streamed row  sblk + 16*(r/8) + 8*lh + r%8.
+  auto block = [&](auto sb_c, auto masked_c, const int sblk, const bool f_ready) __attribute__((always_inline)) {
+    constexpr int sb = decltype(sb_c)::value;
+    constexpr bool masked = decltype(masked_c)::value != 0;
+    constexpr int NSTEP = 2 * K;
+    f32x16 S = (f32x16){0}, dP = (f32x16){0};
+    auto frag = [&](int st) __attribute__((always_inline)) -> i32x4 {
+      return st < K ? fr.rows(0, sb, st) : fr.rows(TILEB, sb, st - K);
+    };
+    auto prob = [&](int r) __attribute__((always_inline)) {   // S[r] <- P[r]
+      S[r] = fast_exp2(fmaf(S[r], scale, -lse_l));
+    };
+    auto dsv = [&](int r) __attribute__((always_inline)) -> float {
+      return S[r] * (dP[r] - delta_l);
+    };
+    if (!f_ready) {
 #pragma unroll
-      for (int st = 0; st < G::KSTEPS; ++st) {
-        S = Elem<T>::mfma(f[st % kPrefetch], Xf[st], S);
-        if (st + kPrefetch < NSTEP) f[st % kPrefetch] = frag(st + kPrefetch);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      // rare: rows / columns that do not exist or lie above the diagonal give P = 0
+      for (int st = 0; st < kPrefetch; ++st) f[st] = frag(st);
+    }
+    // Issue priority: highest while the wave feeds the accumulators (the last
+    // product, 2*NDB MFMAs over NDB independent chains), low during the two
+    // serial chains S and dP; the two waves of a SIMD then fall out of step
+    // instead of competing with the same kind of work (measured 3 %).
+    __builtin_amdgcn_s_setprio(1);
+    static_for<0, K>([&](auto st_c) __attribute__((always_inline)) {
+      constexpr int st = decltype(st_c)::value;
+      S = Elem<T>::mfma(f[st % kPrefetch], Xf[st], S);
+      if (st + kPrefetch < NSTEP) f[st % kPrefetch] = frag(st + kPrefetch);
+      if (sb == 0 && !masked)
+        static_for<0, IPT>([&](auto n_c) __attribute__((always_inline)) {
+          if (st == drip_slice(decltype(n_c)::value)) drip(decltype(n_c)::value);
+        });
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    if (masked) {
+      // rows / columns that do not exist or lie above the diagonal give P = 0
       bool need_mask = sblk + 32 > len;
       if (causal) need_mask = need_mask || sblk + 31 > r0w;
       if (need_mask) {
@@ -314,80 +355,97 @@ __device__ __forceinline__ void bwd_dq_item(const BwdParams& p, const int bid) {
           S[r] = ok ? S[r] : -INFINITY;
         }
       }
-      i32x4 tf[2];
-      uint32_t W[8];
+    }
+    i32x4 tf[2];
+    uint32_t W[8];
 #pragma unroll
-      for (int c = 0; c < G::KSTEPS; ++c) {
-        const int st = G::KSTEPS + c;
-        dP = Elem<T>::mfma(f[st % kPrefetch], Yf[c], dP);
-        if (st + kPrefetch < NSTEP) f[st % kPrefetch] = frag(st + kPrefetch);
-        if (c >= G::KSTEPS - 2) tf[c - (G::KSTEPS - 2)] = fr.tr(TT, 2 * sb, c - (G::KSTEPS - 2));
-        // 16 exponentials spread over the KSTEPS slices
+    for (int c = 0; c < K; ++c) {
+      const int st = K + c;
+      dP = Elem<T>::mfma(f[st % kPrefetch], Yf[c], dP);
+      if (st + kPrefetch < NSTEP) f[st % kPrefetch] = frag(st + kPrefetch);
+      if (c >= K - 2) tf[c - (K - 2)] = fr.tr(0, 2 * sb, c - (K - 2));
+      // 16 exponentials spread over the K slices
 #pragma unroll
-        for (int r = 16 * c / G::KSTEPS; r < 16 * (c + 1) / G::KSTEPS; ++r) prob(r);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) W[i] = Elem<T>::pack2(dsv(2 * i), dsv(2 * i + 1));
+      for (int r = 16 * c / K; r < 16 * (c + 1) / K; ++r) prob(r);
       __builtin_amdgcn_sched_barrier(0);
-      // last product: 2*NDB MFMAs, fragment (kk, db) = step kk*NDB + db
-      constexpr int NACC = 2 * G::NDB;
-      __builtin_amdgcn_s_setprio(3);
+    }
 #pragma unroll
-      for (int i = 0; i < NACC; ++i) {
-        const int kk = i / G::NDB, db = i % G::NDB;
-        const i32x4 wf = {(int)W[4 * kk], (int)W[4 * kk + 1], (int)W[4 * kk + 2], (int)W[4 * kk + 3]};
-        acc[db] = Elem<T>::mfma(tf[i & 1], wf, acc[db]);
-        if (i + 2 < NACC) tf[i & 1] = fr.tr(TT, 2 * sb + (i + 2) / G::NDB, (i + 2) % G::NDB);
-        // the ring is idle now: fetch the first fragments of the tile's second block
-        if (sb == 0 && i >= NACC - kPrefetch) f[i - (NACC - kPrefetch)] = fr.rows(T0, 1, i - (NACC - kPrefetch));
-        if (i < G::NDB) {
-          // second half of dS (8 values) spread over the first NDB slices
+    for (int i = 0; i < 4; ++i) W[i] = Elem<T>::pack2(dsv(2 * i), dsv(2 * i + 1));
+    __builtin_amdgcn_sched_barrier(0);
+    // last product: 2*NDB MFMAs, fragment (kk, db) = step kk*NDB + db
+    constexpr int NACC = 2 * G::NDB;
+    __builtin_amdgcn_s_setprio(3);
 #pragma unroll
-          for (int q = 4 * i / G::NDB; q < 4 * (i + 1) / G::NDB; ++q)
-            W[4 + q] = Elem<T>::pack2(dsv(8 + 2 * q), dsv(9 + 2 * q));
-        }
-        __builtin_amdgcn_sched_barrier(0);
+    for (int i = 0; i < NACC; ++i) {
+      const int kk = i / G::NDB, db = i % G::NDB;
+      const i32x4 wf = {(int)W[4 * kk], (int)W[4 * kk + 1], (int)W[4 * kk + 2], (int)W[4 * kk + 3]};
+      acc[db] = Elem<T>::mfma(tf[i & 1], wf, acc[db]);
+      if (i + 2 < NACC) tf[i & 1] = fr.tr(0, 2 * sb + (i + 2) / G::NDB, (i + 2) % G::NDB);
+      // the ring is idle now: fetch the first fragments of the tile's second block
+      if (sb == 0 && i >= NACC - kPrefetch) f[i - (NACC - kPrefetch)] = fr.rows(0, 1, i - (NACC - kPrefetch));
+      if (i < G::NDB) {
+        // second half of dS (8 values) spread over the first NDB slices
+#pragma unroll
+        for (int q = 4 * i / G::NDB; q < 4 * (i + 1) / G::NDB; ++q)
+          W[4 + q] = Elem<T>::pack2(dsv(8 + 2 * q), dsv(9 + 2 * q));
       }
-      f_ready = sb == 0;
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
+  // a tile whose 64 keys all exist and lie at or before this wave's first query
+  auto compute_fast = [&](int s0) __attribute__((always_inline)) {
+    block(ic<0>{}, ic<0>{}, s0, false);
+    block(ic<1>{}, ic<0>{}, s0 + 32, true);
+  };
+  // a tile on the diagonal or at the sequence end
+  auto compute_slow = [&](int s0) __attribute__((always_inline)) {
+    drip_all();
+    bool f_ready = false;
+    if (s0 < len && !(causal && s0 > r0w + 31)) {
+      block(ic<0>{}, ic<1>{}, s0, false);
+      f_ready = true;
+    }
+    if (s0 + 32 < len && !(causal && s0 + 32 > r0w + 31)) block(ic<1>{}, ic<1>{}, s0 + 32, f_ready);
+  };
 
-  auto step = [&](auto stage_c, int u) __attribute__((always_inline)) {
-    constexpr int ST = decltype(stage_c)::value;
+  // tiles 0 .. NS-2 are requested up front; step u requests tile u + NS - 1
+  // into the stage that tile u - 1 has left
+#pragma unroll
+  for (int u = 0; u < NS - 1; ++u)
+    if (u < n_stream) {
+      request();
+      drip_all();
+      advance();
+    }
+  // resident operands and tile 0 are needed now; the full wait also tells the
+  // compiler that no register load is pending inside the loop
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+  __syncthreads();
+  // Each loop below holds ONE kind of step (with the masked and the unmasked
+  // path in one loop body the accumulators were copied between two register
+  // sets on every trip); every step ends in the workgroup's barrier, so the
+  // waves may split the tiles differently.
+  int n_fast = min(n_stream, len / TN);
+  if (causal) n_fast = min(n_fast, (r0w + 1) / TN);
+  auto step = [&](auto fast_c, int u) __attribute__((always_inline)) {
     const bool refill = u + NS - 1 < n_stream;
-    if (refill) issue(u + NS - 1, ic<(ST + NS - 1) % NS>{});
-    compute(u, stage_c);
+    if (refill) request();
+    if (decltype(fast_c)::value)
+      compute_fast(u * TN);
+    else
+      compute_slow(u * TN);
+    rotate();
+    if (refill) advance();
     // the next tile must have landed (this wave's loads retire in order: only
-    // the tiles requested after it may still fly) and everyone is done with this one
-    const int younger = min(n_stream - 1, u + NS - 1) - (u + 1);
-    if (younger >= 2)
-      __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * IPT));
-    else if (younger == 1)
+    // the tile requested in this step may still fly) and everyone is done with this one
+    if (refill)
       __builtin_amdgcn_s_waitcnt(waitcnt_vm(IPT));
     else
       __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __syncthreads();
   };
-
-  if (n_stream > 0) issue(0, ic<0>{});
-  if (n_stream > 1) issue(1, ic<1>{});
-  if (NS > 3 && n_stream > 2) issue(2, ic<2 % NS>{});
-  // resident operands and tile 0 are needed now; the full wait also tells the
-  // compiler that no register load is pending inside the loop
-  __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-  __syncthreads();
-  for (int u = 0; u < n_stream; u += NS) {
-    step(ic<0>{}, u);
-    if (u + 1 >= n_stream) break;
-    step(ic<1>{}, u + 1);
-    if (u + 2 >= n_stream) break;
-    step(ic<2>{}, u + 2);
-    if (NS > 3) {
-      if (u + 3 >= n_stream) break;
-      step(ic<3 % NS>{}, u + 3);
-    }
-  }
+  for (int u = 0; u < n_fast; ++u) step(ic<1>{}, u);
+  for (int u = n_fast; u < n_stream; ++u) step(ic<0>{}, u);
   __builtin_amdgcn_s_setprio(0);
   __syncthreads();
 
