@@ -126,16 +126,33 @@ __global__ void __launch_bounds__(512) xent_gemm_kernel(const XentParams p) {
   };
   int iss_k = 0, iss_n0 = tile_first * kXTileN;
   set_woff(iss_n0);
-  auto issue = [&](int stage) __attribute__((always_inline)) {
-    const uint64_t wb = w_base + (uint64_t)iss_n0 * w_pitch + (uint32_t)(iss_k * kXStepK * 2);
-    const uint64_t xb = x_base + (uint64_t)t0 * x_pitch + (uint32_t)(iss_k * kXStepK * 2);
-    const uint32_t sw = lds0 + stage * kXSlabB + wave * 4096;
-    const uint32_t sx = lds0 + (2 + stage) * kXSlabB + wave * 4096;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      dma16(wb + woff[q], sw + q * 1024);
-      dma16(xb + xoff[q], sx + q * 1024);
-    }
+  // The eight loads of a step (four of W, four of X per wavefront) are sent one
+  // at a time behind the first MFMAs of the step before: sent together right
+  // after the barrier, 64 KiB of requests queue up in the memory pipeline and a
+  // wavefront reaches its MFMAs only when its own requests have been accepted.
+  // arm() fixes the wave-uniform slab addresses, drip(k) sends load k, next()
+  // moves on; a load whose mask is 0 is a no-op (all 64 lanes are active and
+  // control flow is wave-uniform here, so exec is restored to all ones).
+  uint64_t drip_on = 0, drip_wb = 0, drip_xb = 0;
+  uint32_t drip_sw = 0, drip_sx = 0;
+  auto arm = [&](int stage, bool on) __attribute__((always_inline)) {
+    drip_on = uniform64(on ? ~0ull : 0ull);
+    drip_wb = uniform64(w_base + (uint64_t)iss_n0 * w_pitch + (uint32_t)(iss_k * kXStepK * 2));
+    drip_xb = uniform64(x_base + (uint64_t)t0 * x_pitch + (uint32_t)(iss_k * kXStepK * 2));
+    drip_sw = lds0 + stage * kXSlabB + wave * 4096;
+    drip_sx = lds0 + (2 + stage) * kXSlabB + wave * 4096;
+  };
+  auto drip = [&](int k) __attribute__((always_inline)) {
+    const int q = k >> 1;
+    const uint64_t base = (k & 1) ? drip_xb : drip_wb;
+    const uint32_t off = (k & 1) ? xoff[q] : woff[q];
+    const uint32_t slab = (uint32_t)__builtin_amdgcn_readfirstlane(((k & 1) ? drip_sx : drip_sw) + q * 1024);
+    asm volatile("s_mov_b32 m0, %3\n\ts_mov_b64 exec, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, -1"
+                 :
+                 : "s"(drip_on), "v"(off), "s"(base), "s"(slab)
+                 : "memory");
+  };
+  auto next = [&]() __attribute__((always_inline)) {
     if (++iss_k == nk) {
       iss_k = 0;
       iss_n0 += kXTileN;
@@ -192,6 +209,7 @@ __global__ void __launch_bounds__(512) xent_gemm_kernel(const XentParams p) {
         }
         acc[rb][0] = Elem<T>::mfma(af[s & 1][rb], bf[s & 1][0], acc[rb][0]);
         acc[rb][1] = Elem<T>::mfma(af[s & 1][rb], bf[s & 1][1], acc[rb][1]);
+        if (4 * s + rb < 8) drip(4 * s + rb);   // the first eight slices carry one load each
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -332,12 +350,17 @@ __global__ void __launch_bounds__(512) xent_gemm_kernel(const XentParams p) {
   // number of step pairs.
   int ck = 0, cn0 = tile_first * kXTileN;
   int it = 0;
-  issue(0);
+  arm(0, total > 0);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) drip(k);
+  next();
   auto step = [&](int stage) __attribute__((always_inline)) {
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __syncthreads();
-    if (++it < total) issue(stage ^ 1);
+    const bool more = ++it < total;
+    arm(stage ^ 1, more);
     compute(stage);
+    if (more) next();
   };
   while (it < total) {
     step(0);
