@@ -29,6 +29,10 @@ CASES = [
     ([513, 1024, 31], 4, 1, 128, torch.float16),
     ([700], 6, 2, 96, torch.float16),
     ([512, 100, 65], 4, 1, 64, torch.bfloat16),
+    # lengths on either side of every tile boundary of the two kernels (64-row
+    # streamed tiles, 128 / 256 resident rows): the masked and the unmasked
+    # steps of an item are walked by separate loops
+    ([63, 64, 65, 127, 129, 191, 192, 193, 320, 384, 385], 4, 1, 128, torch.bfloat16),
 ]
 
 
