@@ -75,7 +75,7 @@ struct BwdParams {
   int64_t dl_sb, dl_sh;
   const int32_t* cu;  // null => batched
   int32_t batch, hq, hkv, max_seqlen;
-  int32_t n_rtiles;   // ceil(max_seqlen / 256)
+  int32_t n_rtiles;   // ceil(max_seqlen / 256): resident tiles of the dQ kernel
   int32_t causal;
   float scale;        // log2 domain
   float scale_nat;    // natural base (= scale * ln 2)
@@ -133,7 +133,7 @@ int launch_decode_merge(const DecodeParams& p, int dtype, int head_dim, hipStrea
 // device (hipError_t as int; no allocation).
 constexpr unsigned kDecodeScratchBytes = 32u << 20;
 int decode_static_scratch(void** ptr);
-// delta, dq, dk, dv kernels in that order
+// delta, dQ and dK + dV kernels in that order
 int launch_attn_bwd(const BwdParams& p, int dtype, int head_dim, hipStream_t s);
 // RMSNorm.  x_dtype: 0 bf16, 1 f16, 2 f32; w_dtype: x_dtype or 2.  `vec`: rows
 // can be read in 16-byte chunks (dim a multiple of the chunk, aligned rows,
