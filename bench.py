@@ -600,12 +600,12 @@ def cpu_baseline(name):
         return sorted(ts)[len(ts) // 2]
 
     if name == "dense_causal":
-        B, H, S, D = 1, 16, 8192, 128
+        B, H, S, D = 1, 32, 8192, 128
         q, k, v = (torch.randn((B, H, S, D), generator=g).to(torch.bfloat16) for _ in range(3))
         t = med(lambda: orc.causal_attention(q, k, v))
         flop = 2.0 * B * H * S * (S + 1) * D
         return {"value": flop / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
-                "sample": "torch-CPU bf16 causal softmax(qk^T/sqrt(d))v (tutorial/4.4 oracle) on B=1 H=16 S=8192 D=128 (1/8 of the workload), "
+                "sample": "torch-CPU bf16 causal softmax(qk^T/sqrt(d))v (tutorial/4.4 oracle) on B=1 H=32 S=8192 D=128 (one of the workload's four sequences), "
                           "median of 3; same algorithmic-FLOP formula as the GPU figure",
                 "seconds": t}
     if name == "c1_dense_noncausal_small":
