@@ -1,0 +1,65 @@
+"""Seeded random shapes for the kernels whose tile loops are split into masked
+and unmasked steps (dense backward, block-sparse prefill): ragged lengths on
+either side of the tile sizes, every head_dim, both dtypes, GQA groups, random
+block masks - each case against the CPU oracle."""
+import random
+
+import pytest
+import torch
+
+from oracle import attention_oracle as orc
+from tests.util import cu_from, randn
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = [0, 1, 31, 63, 64, 65, 100, 127, 128, 129, 200, 255, 256, 257, 300, 383, 385, 511, 513, 700]
+
+
+def _rel(got, want):
+    got, want = got.float().cpu(), want.float()
+    assert torch.isfinite(got).all()
+    return (got - want).abs().max().item() / max(want.abs().max().item(), 1.0)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_backward_random_ragged_batches(seed):
+    import tritonops_amd as ta
+
+    rnd = random.Random(seed)
+    lens = [rnd.choice(LENGTHS) for _ in range(rnd.randint(1, 4))]
+    if sum(lens) == 0:
+        lens[0] = 77
+    Hkv = rnd.choice([1, 2, 4])
+    Hq = Hkv * rnd.choice([1, 2, 4])
+    D = rnd.choice([64, 96, 128])
+    dt = rnd.choice([torch.bfloat16, torch.float16])
+    cu = cu_from(torch.tensor(lens, dtype=torch.int32))
+    T = int(cu[-1])
+    q, k, v = randn((1, T, Hq, D), 1 + seed, dt), randn((1, T, Hkv, D), 2 + seed, dt), randn((1, T, Hkv, D), 3 + seed, dt)
+    do = randn((1, T, Hq, D), 4 + seed, dt)
+    want = orc.varlen_masked_attention_backward(q, k, v, do, cu, orc.causal_mask)
+    sm = D ** -0.5 * ta.LOG2E
+    o, lse = ta.flash_attn_triton_fwd(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), sm)
+    got = ta.flash_attn_triton_bwd(q.cuda(), k.cuda(), v.cuda(), o, do.cuda(), lse, cu.cuda(), sm)
+    for name, a, b in zip(("dq", "dk", "dv"), got, want):
+        assert _rel(a, b) <= 3e-2, (name, lens, Hq, Hkv, D, dt)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_block_sparse_prefill_random_masks(seed):
+    import tritonops_amd as ta
+
+    rnd = random.Random(100 + seed)
+    S = rnd.choice([64, 100, 257, 512, 1000, 2048])
+    H = rnd.choice([1, 2, 4])
+    Hkv = rnd.choice([h for h in (1, 2, 4) if H % h == 0])
+    D = rnd.choice([64, 96, 128])
+    dt = rnd.choice([torch.bfloat16, torch.float16])
+    nb = (S + 63) // 64
+    m = torch.rand(nb, nb, generator=torch.Generator().manual_seed(seed)) < rnd.choice([0.1, 0.5, 1.0])
+    m = m.tril() | torch.eye(nb, dtype=torch.bool)
+    cu = cu_from(torch.tensor([S], dtype=torch.int32))
+    q, k, v = randn((1, S, H, D), 10 + seed, dt), randn((1, S, Hkv, D), 11 + seed, dt), randn((1, S, Hkv, D), 12 + seed, dt)
+    want = orc.block_sparse_attention(q, k, v, cu, m)
+    got, _ = ta.flash_attn_sparse_triton(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), None, block_mask=m)
+    assert _rel(got, want) <= 2e-2, (S, H, Hkv, D, dt)
