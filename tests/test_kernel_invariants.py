@@ -84,3 +84,53 @@ def test_q_registers_are_untouched_between_load_and_wait(dense_kernels):
                 if "global_load_dwordx4" in l and "lds" not in l:
                     continue
                 assert not (_regs(l) & q), (dtype, d, i, l.strip())
+
+
+# ---------------------------------------------------------------------------
+# Direct-to-LDS loads with a scalar base, issued from inline assembly.  A vector
+# memory instruction that reads a scalar register written by a VECTOR
+# instruction needs five wait states between the two, and the compiler cannot
+# see into an assembly statement to add them.  The kernels therefore form every
+# such base with scalar arithmetic (or read it to a scalar register well
+# before); this checks the generated code of every kernel that uses the form.
+@pytest.fixture(scope="module")
+def saddr_sources(tmp_path_factory):
+    if not os.path.exists(HIPCC):
+        pytest.skip("hipcc not available")
+    out_dir = tmp_path_factory.mktemp("asm_all")
+    texts = {}
+    procs = []
+    for name in ("prefill.hip", "bwd.hip", "xent.hip"):
+        out = out_dir / (name + ".s")
+        cmd = [HIPCC, "-x", "hip", "--offload-arch=gfx950", "-O3", "-std=c++17",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               "-I", os.path.join(ROOT, "include"), "--cuda-device-only", "-S",
+               os.path.join(ROOT, "tritonops_amd", "csrc", name), "-o", str(out)]
+        procs.append((name, out, subprocess.Popen(cmd, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)))
+    for name, out, proc in procs:
+        assert proc.wait() == 0, name
+        texts[name] = out.read_text()
+    return texts
+
+
+def test_scalar_bases_of_lds_loads_are_not_fresh_vector_results(saddr_sources):
+    n_loads = 0
+    for name, text in saddr_sources.items():
+        lines = [l for l in text.split("\n")
+                 if l.strip() and not l.strip().startswith(";") and not l.strip().startswith(".")]
+        for k, line in enumerate(lines):
+            m = re.search(r"global_load_lds_dword(?:x4)? v\d+, s\[(\d+):(\d+)\]", line)
+            if not m:
+                continue
+            n_loads += 1
+            lo, hi = int(m.group(1)), int(m.group(2))
+            for back in range(1, 7):
+                prev = lines[k - back]
+                if prev.strip().endswith(":"):
+                    break
+                w = re.match(r"\s*(v_\S+)\s+s\[(\d+):(\d+)\]", prev) or re.match(r"\s*(v_\S+)\s+s(\d+)\b", prev)
+                if w:
+                    d0 = int(w.group(2))
+                    d1 = int(w.group(3)) if (w.lastindex or 0) >= 3 else d0
+                    assert not (d0 <= hi and d1 >= lo), (name, k, prev.strip(), line.strip())
+    assert n_loads > 100   # the form is in use (dense forward, both backward kernels, cross-entropy)
