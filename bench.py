@@ -45,7 +45,7 @@ KERNELS = {
     "block_sparse": _NS + "13sparse_kernelIDF16bLi128ELi2ELi2ELi32EEEvNS_13PrefillParamsE",
     "sparse_decode": _NS + "21decode_splitkv_kernelIDF16bLi128EEEvNS_12DecodeParamsE",
     "dense_causal_bwd": " + ".join(_NS + n for n in (
-        "16bwd_delta_kernelIDF16bEEvNS_9BwdParamsEi", "13bwd_dq_kernelIDF16bLi128EEEvNS_9BwdParamsEi",
+        "13bwd_dq_kernelIDF16bLi128EEEvNS_9BwdParamsEi",
         "15bwd_dkdv_kernelIDF16bLi128EEEvNS_9BwdParamsEii")),
     "rmsnorm": " + ".join(_NS + n for n in (
         "18rms_fwd_vec_kernelIDF16bfLi2ELi4EEEvNS_9RmsParamsE", "18rms_bwd_vec_kernelIDF16bfLi2ELi4EEEvNS_9RmsParamsE",
@@ -241,7 +241,7 @@ def run_dense_bwd(steps, warmup):
                      "unit": "TFLOP/s", "kernel": KERNELS["dense_causal_bwd"]},
         "config": {"workload": "dense causal attention bwd bf16 B=4 H=32 S=8192 D=128: dq, dk, dv from q, k, v, o, lse, do",
                    "flop_per_step": flop,
-                   "note": "delta, dq and a fused dk + dv kernel execute 14*D FLOP per pair (S and dP twice); the figure "
+                   "note": "a dq kernel (which also forms delta) and a fused dk + dv kernel execute 14*D FLOP per pair (S and dP twice); the figure "
                            "counts the 10*D of a single-pass backward"},
     }
 

@@ -109,7 +109,7 @@ int mi_attn_fwd(const mi_attn_fwd_args *args, void *stream);
  * (dtype as q; dk/dv have heads_kv heads: the query heads of a GQA group are
  * summed inside the kernel).  Addressing modes, causal flag and scale as in
  * mi_attn_fwd.  The workspace holds
- * Delta = rowsum(o * dout) in fp32.  Four launches on `stream`.
+ * Delta = rowsum(o * dout) in fp32.  Two launches on `stream`.
  */
 typedef struct mi_attn_bwd_args {
   uint32_t struct_size;

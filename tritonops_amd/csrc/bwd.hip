@@ -18,6 +18,8 @@
 // the other side through a three-stage LDS ring (direct-to-LDS loads).
 //   dQ     : resident q, do rows; streams K, V.
 //            S^T = K Q^T, dP^T = V dO^T, dQ^T += K^T dS^T
+//            It also forms Delta of its resident rows (one pass over the o
+//            rows) and stores it for the second kernel, which runs after it.
 //   dK + dV: resident k, v rows; streams Q, dO (all query heads of the GQA
 //            group in turn).  The work of a 32-row group is split between two
 //            wavefronts that share a SIMD: one forms S, P and dV^T += dO^T P,
@@ -174,14 +176,25 @@ __device__ __forceinline__ void bwd_dq_item(const BwdParams& p, const int bid) {
   // ---- resident B operands: lane (row lq, half lh) holds d = 16c + 8lh .. +7
   const T* xp = reinterpret_cast<const T*>(p.q) + bsel * p.q_sb + (start + rclamp) * p.q_ss + hr * p.q_sh;
   const T* yp = reinterpret_cast<const T*>(p.dout) + bsel * p.do_sb + (start + rclamp) * p.do_ss + hr * p.do_sh;
+  const T* op = reinterpret_cast<const T*>(p.o) + bsel * p.o_sb + (start + rclamp) * p.o_ss + hr * p.o_sh;
   i32x4 Xf[G::KSTEPS], Yf[G::KSTEPS];
+  // Delta[row] = sum_d o[row][d] * do[row][d] (fp32) is formed here, from the
+  // resident do rows and one pass over the o rows, and stored for the dK + dV
+  // kernel, which runs after this one.
+  float delta_l = 0.f;
 #pragma unroll
   for (int c = 0; c < G::KSTEPS; ++c) {
     Xf[c] = *reinterpret_cast<const i32x4*>(xp + 8 * fr.lh + 16 * c);
     Yf[c] = *reinterpret_cast<const i32x4*>(yp + 8 * fr.lh + 16 * c);
+    const i32x4 Of = *reinterpret_cast<const i32x4*>(op + 8 * fr.lh + 16 * c);
+    const T* oe = reinterpret_cast<const T*>(&Of);
+    const T* de = reinterpret_cast<const T*>(&Yf[c]);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) delta_l += (float)oe[i] * (float)de[i];
   }
+  delta_l += __shfl_xor(delta_l, 32);
+  if (fr.lh == 0 && rrow < len) p.delta[(int64_t)b * p.dl_sb + (int64_t)hr * p.dl_sh + rrow] = delta_l;
   const float lse_l = p.lse[bsel * p.lse_sb + (start + rclamp) * p.lse_ss + hr * p.lse_sh];
-  const float delta_l = p.delta[(int64_t)b * p.dl_sb + (int64_t)hr * p.dl_sh + rclamp];
 
   f32x16 acc[G::NDB];
 #pragma unroll
@@ -1096,39 +1109,6 @@ bwd_dq_kernel(const BwdParams p, const int n_items) {
   }
 }
 
-// Delta[b][h][s] = sum_d o[s][d] * do[s][d], fp32.  16 lanes per row (one 16-byte
-// chunk each), 16 rows per 256-thread workgroup.
-template <typename T>
-__global__ void __launch_bounds__(256) bwd_delta_kernel(const BwdParams p, int head_dim) {
-  const int ch = threadIdx.x & 15;
-  const int row = blockIdx.x * 16 + (threadIdx.x >> 4);
-  const int h = blockIdx.y, b = blockIdx.z;
-  int len;
-  int64_t start;
-  if (p.cu) {
-    start = p.cu[b];
-    len = p.cu[b + 1] - (int)start;
-  } else {
-    start = 0;
-    len = p.max_seqlen;
-  }
-  const int64_t bsel = p.cu ? 0 : b;
-  float s = 0.f;
-  if (row < len && ch * 8 < head_dim) {
-    const T* op = reinterpret_cast<const T*>(p.o) + bsel * p.o_sb + (start + row) * p.o_ss + h * p.o_sh + ch * 8;
-    const T* dp = reinterpret_cast<const T*>(p.dout) + bsel * p.do_sb + (start + row) * p.do_ss + h * p.do_sh + ch * 8;
-    const i32x4 ov = *reinterpret_cast<const i32x4*>(op);
-    const i32x4 dv = *reinterpret_cast<const i32x4*>(dp);
-    const T* oe = reinterpret_cast<const T*>(&ov);
-    const T* de = reinterpret_cast<const T*>(&dv);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) s += (float)oe[i] * (float)de[i];
-  }
-#pragma unroll
-  for (int m = 8; m >= 1; m >>= 1) s += __shfl_xor(s, m, 16);
-  if (ch == 0 && row < len) p.delta[(int64_t)b * p.dl_sb + (int64_t)h * p.dl_sh + row] = s;
-}
-
 template <typename T, int D>
 int launch_dq(const BwdParams& p, hipStream_t s) {
   constexpr size_t lds = kBwdStages * (2 * 64 * 256 + 1024);
@@ -1162,10 +1142,8 @@ int launch_dkdv(const BwdParams& p, hipStream_t s) {
 
 template <typename T, int D>
 int launch_all(const BwdParams& p, hipStream_t s) {
-  dim3 grid((p.max_seqlen + 15) / 16, p.hq, p.batch);
-  hipLaunchKernelGGL((bwd_delta_kernel<T>), grid, dim3(256), 0, s, p, D);
-  int rc = (int)hipGetLastError();
-  if (rc) return rc;
+  // dQ first: it also writes Delta, which the dK + dV kernel reads
+  int rc;
   if ((rc = launch_dq<T, D>(p, s))) return rc;
   return launch_dkdv<T, D>(p, s);
 }

@@ -133,7 +133,7 @@ int launch_decode_merge(const DecodeParams& p, int dtype, int head_dim, hipStrea
 // device (hipError_t as int; no allocation).
 constexpr unsigned kDecodeScratchBytes = 32u << 20;
 int decode_static_scratch(void** ptr);
-// delta, dQ and dK + dV kernels in that order
+// the dQ kernel (which also writes Delta), then the dK + dV kernel
 int launch_attn_bwd(const BwdParams& p, int dtype, int head_dim, hipStream_t s);
 // RMSNorm.  x_dtype: 0 bf16, 1 f16, 2 f32; w_dtype: x_dtype or 2.  `vec`: rows
 // can be read in 16-byte chunks (dim a multiple of the chunk, aligned rows,
