@@ -531,9 +531,11 @@ sparse_kernel(const PrefillParams p) {
 //
 // Item boundary: once every wave is done with the tiles of an item, the
 // workgroup requests Q and the first NS-1 tiles of its NEXT item (stages
-// 0..NS-2) and only then normalises and writes out the current one, staging
-// the output through the last stage, so the load latency of the next item is
-// covered by the epilogue of this one; one barrier separates the two items.
+// 0..NS-2) while it normalises and writes out the current one, staging the
+// output through the last stage: Q and tile 0 go out first, tiles 1 and 2
+// after the first and the second pass of output stores, so the requests queue
+// in the vector-memory pipeline while the waves do the arithmetic of the
+// write-out instead of in front of it; one barrier separates the two items.
 //
 // Inner loop: a software pipeline over HALF tiles (32 keys) inside each wave.
 // MFMA and softmax arithmetic overlap best when one wave's instruction stream
@@ -603,7 +605,7 @@ dense_kernel(const PrefillParams p) {
     return false;
   };
   // Q^T operands of an item (lane (query lq, half lh) holds d = 16c + 8lh .. +7)
-  // and its first NS-1 tiles; nothing waits here
+  // and its first tile (tiles 1 and 2 follow from request_tile1 / 2); nothing waits here
   auto request_item = [&](const Item& it, i32x4 (&Q)[G::KSTEPS]) __attribute__((always_inline)) {
     const int row = min(it.q0 + 32 * rblk + fr.lq, it.len - 1);
     const T* qr = it.qp + (int64_t)row * p.q_ss + 8 * fr.lh;
@@ -615,7 +617,11 @@ dense_kernel(const PrefillParams p) {
     for (int c = 0; c < G::KSTEPS; ++c)
       asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(Q[c]) : "v"(qr), "n"(32 * c));
     if (0 < it.n_tiles) dma.template tile<0>(it.kv, 0);
+  };
+  auto request_tile1 = [&](const Item& it) __attribute__((always_inline)) {
     if (1 < it.n_tiles) dma.template tile<1>(it.kv, TN);
+  };
+  auto request_tile2 = [&](const Item& it) __attribute__((always_inline)) {
     if (2 < it.n_tiles) dma.template tile<2>(it.kv, 2 * TN);
   };
 
@@ -786,7 +792,7 @@ dense_kernel(const PrefillParams p) {
   // 16-byte store instructions a wave issues for 32 rows that all exist; they
   // are the last vector-memory instructions of an item
   constexpr int kOutStores = 2 * (32 * CH / 64);
-  auto write_out = [&]() __attribute__((always_inline)) {
+  auto write_out = [&](auto&& after_pass0, auto&& after_pass1) __attribute__((always_inline)) {
     static_assert(4 * 32 * SROW <= TILEB, "four waves stage inside one tile");
     auto sswz = [](int row) { return SROW == 128 ? ((row >> 1) & 7) : ((row >> 2) & 3); };
     // Lane coordinates through an opaque copy: the staging and output offsets
@@ -834,11 +840,19 @@ dense_kernel(const PrefillParams p) {
         }
       }
       asm volatile("" ::: "memory");
+      if (ps == 0)
+        after_pass0();
+      else
+        after_pass1();
     }
   };
 
   bool have = next_item(cur);
-  if (have) request_item(cur, Qf);
+  if (have) {
+    request_item(cur, Qf);
+    request_tile1(cur);
+    request_tile2(cur);
+  }
   int out_stores = 0;  // output stores of the previous item that may still be in flight
   while (have) {
     len = cur.len;
@@ -857,17 +871,18 @@ dense_kernel(const PrefillParams p) {
     m_neg = 0.f;
     l = 0.f;
 
-    // Every load requested so far must have landed: the Q operands and tile 0
-    // are needed now, and a wait that covers all register loads also tells the
-    // compiler that none is pending inside the loop (it would otherwise guard
-    // the first use of every Q register there with a wait that also drains the
-    // tile loads).  The only younger instructions are the output stores of the
-    // previous item, which may stay in flight: vmcnt retires loads and stores
-    // in issue order, and out_stores is a lower bound of their number.  The
+    // The Q operands and tiles 0 and 1 must have landed (K of tile 1 is read
+    // while tile 0 is finished).  At an item boundary the requests and the
+    // previous item's output stores were issued in the order
+    //   Q, tile 0, stores of pass 0, tile 1, stores of pass 1, tile 2
+    // so that the loads queue behind one another while the wave works on the
+    // write-out.  vmcnt retires loads and stores in issue order: the stores of
+    // pass 1 and the loads of tile 2 may stay in flight when both were issued
+    // in full (out_stores says so); otherwise everything is waited for.  The
     // barrier publishes the tiles and separates the previous item's staging
     // reads from the refill of the last stage, which follows at once.
     if (out_stores == kOutStores)
-      __builtin_amdgcn_s_waitcnt(waitcnt_vm(kOutStores));
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm(kOutStores / 2 + 2 * IPW));
     else
       __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     // The Q registers were written by loads the compiler cannot see.  Passing
@@ -912,8 +927,10 @@ dense_kernel(const PrefillParams p) {
     Item nxt = cur;
     const bool more = next_item(nxt);
     if (more) request_item(nxt, Qf);  // (Qf is dead by now; no copy may sit between a load and its wait)
-    write_out();
-    out_stores = (q0w + 32 <= len) ? kOutStores : 0;  // every store instruction had live lanes
+    write_out([&]() __attribute__((always_inline)) { if (more) request_tile1(nxt); },
+              [&]() __attribute__((always_inline)) { if (more) request_tile2(nxt); });
+    // every store instruction had live lanes and tile 2 was requested behind them
+    out_stores = (q0w + 32 <= len && more && 2 < nxt.n_tiles) ? kOutStores : 0;
     cur = nxt;
     have = more;
   }
