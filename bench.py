@@ -42,7 +42,7 @@ KERNELS = {
     "dense_causal": _NS + "12dense_kernelIDF16bLi128EEEvNS_13PrefillParamsE",
     "c1_dense_noncausal_small": _NS + "12dense_kernelIDF16bLi64EEEvNS_13PrefillParamsE",
     "gqa_decode": _NS + "21decode_splitkv_kernelIDF16bLi128EEEvNS_12DecodeParamsE",
-    "block_sparse": _NS + "13sparse_kernelIDF16bLi128ELi2ELi2ELi32EEEvNS_13PrefillParamsE",
+    "block_sparse": _NS + "13sparse_kernelIDF16bLi128EEEvNS_13PrefillParamsE",
     "sparse_decode": _NS + "21decode_splitkv_kernelIDF16bLi128EEEvNS_12DecodeParamsE",
     "dense_causal_bwd": " + ".join(_NS + n for n in (
         "13bwd_dq_kernelIDF16bLi128EEEvNS_9BwdParamsEi",

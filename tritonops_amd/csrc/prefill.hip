@@ -5,11 +5,11 @@
 // rows of one (sequence, q-head); KV is walked in tiles that the whole
 // workgroup brings into an LDS ring with direct-to-LDS loads
 // (global_load_lds_dwordx4: no staging registers, no ds_write), one barrier
-// per tile.  Block-sparse: 32-key tiles, two stages, one launch per item, each
-// wavefront runs compute_tile() on its 32 rows.  Dense: 64-key tiles, four
-// stages, a persistent grid that walks the items and requests the first tiles
-// of its next item before it writes out the current one, and a software
-// pipeline over half tiles inside each wavefront (see dense_kernel).
+// per tile.  Dense: 64-key tiles, four stages, a persistent grid that walks the
+// items and requests the first tiles of its next item while it writes out the
+// current one, and a software pipeline over half tiles inside each wavefront
+// (see dense_kernel).  Block-sparse: the same pipeline over 32-key tiles of
+// the listed blocks, two stages per tensor, one launch per item.
 //
 // Replaces flash_attn_fwd_kernel of flash_attn_triton/flash_attn_triton.py
 // :52-180 (dense) and flash_attn_triton/flash_attn_sparse_attn_triton.py
@@ -223,6 +223,26 @@ struct TileDma {
     return s;
   }
 
+  // keys k0 .. k0+TN-1 of K (or of V) into stage ST, rows past the sequence
+  // end re-reading its last row
+  template <int ST, bool IS_V>
+  __device__ __forceinline__ void tensor_tile(const KvSrc<T>& s, int k0) const {
+    const uint32_t sB = lds0 + (IS_V ? VBASE : 0) + ST * TILEB;
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    const int drow = ln / F::SLOTS, dslot = ln % F::SLOTS;
+    const int64_t rowb = IS_V ? v_rowb : k_rowb;
+    const char* bt = reinterpret_cast<const char*>(IS_V ? s.vp : s.kp) + k0 * rowb;
+#pragma unroll
+    for (int t = 0; t < IPW; ++t) {
+      const int inst = wave + NW * t;
+      const int r = RPI * inst + drow;
+      const int c = dslot ^ (IS_V ? F::swz_v(r) : F::swz_k(r));
+      const int64_t rr = min(k0 + r, s.len - 1) - k0;
+      if (D != 96 || c < G::NCH) dma16(bt + rr * rowb + c * 16, sB + inst * 1024);
+    }
+  }
+
   // keys k0 .. k0+TN-1 of `s` into stage ST
   template <int ST>
   __device__ __forceinline__ void tile(const KvSrc<T>& s, int k0) const {
@@ -272,11 +292,31 @@ struct TileDma {
 };
 
 // ---------------------------------------------------------------------------
-// Block-sparse: one workgroup of NW wavefronts per q tile of 32*NW rows (one
-// block row), TN-key tiles of the listed blocks through an NS-stage ring.
-template <typename T, int D, int NW, int NS, int TN>
-__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2)))
+// Block-sparse: one workgroup of two wavefronts per 64-row block row, four
+// workgroups per CU, the dense kernel's software pipeline (see dense_kernel
+// below) over the 32-key tiles of the listed blocks.  At position h a wave runs
+//   block A: [MFMAs of S(h+1) = K(h+1) Q^T]  with [exp2 / sum / pack of the last 8 keys of S(h)]
+//                                             and the loads of K(h+2) and V(h+1), one per MFMA
+//   check  : row sums sane? else exact_fix (rare); mask S(h+1) if its tile needs one
+//   block B: [MFMAs of O += V(h)^T P(h)^T]   with [exp2 / sum / pack of the first 8 keys of S(h+1)]
+// K tiles live one position ahead of V tiles, so each tensor has a ring of its
+// own two stages: K(h+2) replaces K(h), which was scored in position h-1, and
+// V(h+1) replaces V(h-1).  One wait and one barrier per position publish both.
+// The loads sit in block A, whose MFMAs form one serial chain and leave the
+// wave time to queue them; behind the four independent chains of block B they
+// measured 6 % slower.  Probabilities are taken against the reference point
+// the row already has (no row maximum in the common path, as in the dense
+// kernel); a row that has not met a visible key yet takes the exact path.
+// The block list is kept in registers, 64 entries at a time (lane l holds
+// entry 64 * chunk + l; the chunk being walked and the one behind it), and
+// read with v_readlane: a memory load inside the tile loop would have to be
+// waited for with vmcnt(0), which also drains the tiles requested a moment
+// ago.  A block's two tiles share one list lookup and one address product.
+template <typename T, int D>
+__global__ void __launch_bounds__(kSparseRows * 2) __attribute__((amdgpu_waves_per_eu(2)))
 sparse_kernel(const PrefillParams p) {
+  constexpr int NW = kSparseRows / 32, NS = kSparseStages, TN = kSparseTileKeys;
+  static_assert(NW == 2 && NS == 2 && TN == 32 && kTileN == 64, "a listed block is two tiles; two stages per tensor");
   using G = RowGeom<D>;
   using F = SwizzledFrags<D>;
   using DMA = TileDma<T, D, NW, NS, TN>;
@@ -290,10 +330,10 @@ sparse_kernel(const PrefillParams p) {
 
   ItemGeo g;
   if (!item_geo<BM>(p, blockIdx.x, g)) return;
-  const int len = g.len, qt = g.qt, h = g.h;
+  const int len = g.len, qt = g.qt, hd = g.h;
   const int q0 = qt * BM;
-  const T* qp = reinterpret_cast<const T*>(p.q) + g.q_off + h * p.q_sh;
-  T* op = reinterpret_cast<T*>(p.o) + g.o_off + h * p.o_sh;
+  const T* qp = reinterpret_cast<const T*>(p.q) + g.q_off + hd * p.q_sh;
+  T* op = reinterpret_cast<T*>(p.o) + g.o_off + hd * p.o_sh;
 
   F fr;
   fr.init(lane, (uint32_t)(uintptr_t)smem, VBASE);
@@ -304,32 +344,18 @@ sparse_kernel(const PrefillParams p) {
   const int q0w = q0 + 32 * wave;
   const int qrow = q0w + fr.lq;
 
-  // ---- tile list: a listed 64-key block is walked as kTileN / TN tiles
-  const int32_t* rp = p.row_ptr + g.b * p.rp_sb + h * p.rp_sh;
-  // (values loaded through vector memory: tell the compiler they are uniform)
+  // ---- tile list: 64 entries at a time in registers
+  const int32_t* rp = p.row_ptr + g.b * p.rp_sb + hd * p.rp_sh;
   const int beg = __builtin_amdgcn_readfirstlane(rp[qt]);
-  const int n_tiles = __builtin_amdgcn_readfirstlane(rp[qt + 1] - beg) * (kTileN / TN);
-  const int32_t* cols = p.col_idx + g.b * p.ci_sb + h * p.ci_sh + beg;
-  // The block list is kept in registers, 64 entries at a time (lane l holds
-  // entry 64 * chunk + l; the chunk being walked and the one behind it), and
-  // read with v_readlane.  A memory load inside the tile loop would have to be
-  // waited for with vmcnt(0), which also drains the tile that was requested a
-  // moment ago: the ring would never have a load in flight during a compute.
-  const int n_blk = n_tiles / (kTileN / TN);
+  const int n_blk = __builtin_amdgcn_readfirstlane(rp[qt + 1] - beg);
+  const int n_tiles = n_blk * 2;
+  const int32_t* cols = p.col_idx + g.b * p.ci_sb + hd * p.ci_sh + beg;
   auto load_cols = [&](int chunk) __attribute__((always_inline)) -> int {
     const int idx = chunk * 64 + lane;
     return idx < n_blk ? cols[idx] : 0;
   };
   int col_chunk = 0;
   int col_cur = load_cols(0), col_nxt = load_cols(1);
-  // first key of tile `it` (it lies in the chunk being walked or in the next one)
-  auto tile_k0 = [&](int it) __attribute__((always_inline)) -> int {
-    constexpr int PER = kTileN / TN;
-    const int q = it / PER;
-    const int v = (q >> 6) == col_chunk ? col_cur : col_nxt;
-    return __builtin_amdgcn_readlane(v, q & 63) * kTileN + (it % PER) * TN;
-  };
-
   // ---- Q^T operands: lane (query lq, half lh) holds d = 16c + 8lh .. +7
   i32x4 Qf[G::KSTEPS];
   {
@@ -341,157 +367,224 @@ sparse_kernel(const PrefillParams p) {
   f32x16 O[G::NDB];
 #pragma unroll
   for (int db = 0; db < G::NDB; ++db) O[db] = (f32x16){0};
-  float m = -INFINITY, l = 0.f;
+  float m = -INFINITY, m_neg = 0.f, l = 0.f;
+  const float scale = p.scale;
+  const int causal = p.causal;
+  const int wl = p.win_local, wg = p.win_global;
 
-  auto step = [&](auto stage_c, int it) {
-    constexpr int ST = decltype(stage_c)::value;
-    if (((it / (kTileN / TN)) >> 6) != col_chunk) {  // walked into the next 64 entries of the list
-      ++col_chunk;
-      col_cur = col_nxt;
-      col_nxt = load_cols(col_chunk + 1);
+  // keys of the tile at k0 that this lane's query must not see -> -inf.
+  // Register r of a score block is key k0 + 8 lh + e(r), e(r) = 16 (r / 8) + r % 8:
+  // every test is "e(r) against a per-lane bound", branch-free.
+  const int lim_row = min(len - 1, causal ? qrow : 0x3fffffff) - 8 * fr.lh;  // largest visible key, less the lane's offset
+  auto mask_tile = [&](int k0, f32x16& Sx) __attribute__((always_inline)) {
+    bool need = (k0 + TN > len) || (causal && k0 + TN - 1 > q0w);
+    if (wl >= 0) need = need || !((k0 + TN - 1 < wg) || (q0w + 31 - k0 < wl));
+    if (need) {
+      const int hi = lim_row - k0;                    // e(r) <= hi
+      const int lo = qrow - wl - 8 * fr.lh - k0;      // window: e(r) > lo ...
+      const int gl = wg - 8 * fr.lh - k0;             // ... or e(r) < gl
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int e = 16 * (r >> 3) + (r & 7);
+        bool ok = e <= hi;
+        if (wl >= 0) ok = ok & ((e > lo) | (e < gl));
+        Sx[r] = ok ? Sx[r] : -INFINITY;
+      }
     }
-    // refill the stage that was read in the previous iteration: a tile that
-    // reaches past the sequence end at once (clamped rows), a whole tile one
-    // load at a time behind the MFMAs of the score chain below.  (Sent in
-    // one go right after the barrier, the eight loads of a wave queue up in
-    // the memory pipeline behind the other waves' and the wave reaches its
-    // arithmetic hundreds of cycles later.)
-    const bool refill = it + NS - 1 < n_tiles;
-    const int k0r = refill ? tile_k0(it + NS - 1) : 0;
-    const bool whole = k0r + TN <= len;
-    if (refill && !whole) dma.template tile<(ST + NS - 1) % NS>(kv, k0r);
-    const typename DMA::Drip drip = dma.template arm<(ST + NS - 1) % NS>(kv, k0r, refill && whole);
-
-    const int k0 = tile_k0(it);
-    // whole tile above the diagonal for this wave: nothing to add
-    const bool skip = p.causal && k0 > q0w + 31;
-    if (!skip) {
-      bool need_mask = (k0 + TN > len) || (p.causal && k0 + TN - 1 > q0w);
-      const int wl = p.win_local, wg = p.win_global;
-      if (wl >= 0) need_mask = need_mask || !((k0 + TN - 1 < wg) || (q0w + 31 - k0 < wl));
-      const int causal = p.causal;
-      auto allowed = [&](int key_in_tile) -> bool {
-        const int key = k0 + key_in_tile;
-        bool ok = key < len && (!causal || key <= qrow);
-        if (wl >= 0) ok = ok && ((qrow - key < wl) || (key < wg));
-        return ok;
-      };
-      // V addresses carry VBASE inside the lane offsets (see fr.init)
-      static_assert(TN == 32, "one 32-key block per tile");
-      constexpr uint32_t sK = ST * TILEB, sV = ST * TILEB;
-      f32x16 S[1];
-      uint32_t P[1][8];
-      {
-        constexpr int kPrefetch = 4;
-        i32x4 kf[kPrefetch];
-#pragma unroll
-        for (int c = 0; c < kPrefetch; ++c) kf[c] = fr.load_k(sK, 0, c);
-        S[0] = (f32x16){0};
-#pragma unroll
-        for (int c = 0; c < G::KSTEPS; ++c) {
-          S[0] = Elem<T>::mfma(kf[c % kPrefetch], Qf[c], S[0]);
-          if (c + kPrefetch < G::KSTEPS) kf[c % kPrefetch] = fr.load_k(sK, 0, c + kPrefetch);
-#pragma unroll
-          for (int k = c * 2 * IPW / G::KSTEPS; k < (c + 1) * 2 * IPW / G::KSTEPS; ++k) dma.one(drip, k);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-      // Online softmax as in softmax_tile(), with the second half of the
-      // exponentials behind the first MFMAs of O^T += V^T P^T (those need the
-      // probabilities of the lane's first eight keys only) and the V
-      // fragments read two MFMAs ahead.
-      i32x4 vf[2];
-      vf[0] = fr.load_v(sV, 0, 0);
-      vf[1] = fr.load_v(sV, 0, 1 % G::NDB);
-      if (need_mask) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int key = 16 * (r >> 3) + 8 * fr.lh + (r & 7);
-          if (!allowed(key)) S[0][r] = -INFINITY;
-        }
-      }
-      float mx = S[0][0];
-#pragma unroll
-      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, S[0][r]);
-      mx = max_with_other_half(mx);
-      const float m_new = fmaxf(m, mx * p.scale);
-      if (__builtin_amdgcn_ballot_w64(m_new > m + kRescaleSlack) != 0) {
-        const float alpha = fast_exp2(m - ((m_new == -INFINITY) ? 0.f : m_new));
-        l *= alpha;
-#pragma unroll
-        for (int db = 0; db < G::NDB; ++db) O[db] *= alpha;
-        m = m_new;
-      }
-      const float m_use = (m == -INFINITY) ? 0.f : m;
-      const float sc = p.scale;
-      float rs = 0.f;
-      auto expo = [&](int i) __attribute__((always_inline)) {
-        const float p0 = fast_exp2(fmaf(S[0][2 * i], sc, -m_use));
-        const float p1 = fast_exp2(fmaf(S[0][2 * i + 1], sc, -m_use));
-        rs += p0 + p1;
-        P[0][i] = Elem<T>::pack2(p0, p1);
-        asm volatile("" : "+v"(P[0][i]));
-      };
-#pragma unroll
-      for (int i = 0; i < 4; ++i) expo(i);
-      __builtin_amdgcn_sched_barrier(0);
-      constexpr int NACC = 2 * G::NDB;
-#pragma unroll
-      for (int i = 0; i < NACC; ++i) {
-        const int kk = i / G::NDB, db = i % G::NDB;
-        const i32x4 pf = {(int)P[0][4 * kk], (int)P[0][4 * kk + 1], (int)P[0][4 * kk + 2], (int)P[0][4 * kk + 3]};
-        O[db] = Elem<T>::mfma(vf[i & 1], pf, O[db]);
-        if (i + 2 < NACC) vf[i & 1] = fr.load_v(sV, (i + 2) / G::NDB, (i + 2) % G::NDB);
-#pragma unroll
-        for (int j = 4 + i * 4 / G::NDB; j < 4 + (i + 1) * 4 / G::NDB; ++j)
-          if (i < G::NDB) expo(j);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      l += rs;
-    } else {
-#pragma unroll
-      for (int k = 0; k < 2 * IPW; ++k) dma.one(drip, k);
-    }
-    // The next tile must have landed and everyone must be done with this one.
-    // This wave's loads complete in order, so it is enough that at most the
-    // loads of the NS-2 younger tiles are still in flight (2*IPW each).
-    if (refill)
-      __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * 2 * IPW));
-    else
-      __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-    __syncthreads();
   };
 
+  constexpr float kRowSumLimit = 4096.f;
+  f32x16 S[2];
+  uint32_t Pb[2][8];
+  float rsv[2];
+  float e_p0, e_u1;
+  auto exp_first = [&](const f32x16& Sx, int i) __attribute__((always_inline)) {
+    e_p0 = fast_exp2(fmaf(Sx[2 * i], scale, m_neg));
+    e_u1 = fmaf(Sx[2 * i + 1], scale, m_neg);
+  };
+  auto exp_second = [&](int i, uint32_t (&Pd)[8], float& rs) __attribute__((always_inline)) {
+    const float p1 = fast_exp2(e_u1);
+    rs = i == 0 ? e_p0 + p1 : rs + (e_p0 + p1);
+    Pd[i] = Elem<T>::pack2(e_p0, p1);
+  };
+  // rare: bring m to the exact running maximum including the tile in Sx,
+  // rescale l and O, and redo the probabilities of that tile
+  auto exact_fix = [&](const f32x16& Sx, uint32_t (&Pd)[8], float& rs) __attribute__((always_inline)) {
+    float mx = Sx[0];
 #pragma unroll
-  for (int s0 = 0; s0 < NS - 1; ++s0)
-    if (s0 < n_tiles) {
-      if (s0 == 0) dma.template tile<0>(kv, tile_k0(0));
-      if (s0 == 1) dma.template tile<1 % NS>(kv, tile_k0(1));
-      if (s0 == 2) dma.template tile<2 % NS>(kv, tile_k0(2));
+    for (int r = 1; r < 16; ++r) mx = fmaxf(mx, Sx[r]);
+    mx = max_with_other_half(mx);
+    const float m_new = fmaxf(m, mx * scale);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = fast_exp2(m - m_safe);
+    l *= alpha;
+#pragma unroll
+    for (int db = 0; db < G::NDB; ++db) O[db] *= alpha;
+    m = m_new;
+    m_neg = -m_safe;
+    rs = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float p0 = fast_exp2(fmaf(Sx[2 * i], scale, -m_safe));
+      const float p1 = fast_exp2(fmaf(Sx[2 * i + 1], scale, -m_safe));
+      rs += p0 + p1;
+      Pd[i] = Elem<T>::pack2(p0, p1);
     }
-  // tile 0 (and the Q loads issued before it) must be complete
-  if (n_tiles >= NS - 1)
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * 2 * IPW));
-  else
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-  __syncthreads();
+  };
 
-  int it = 0;
-  for (; it + NS <= n_tiles; it += NS) {
-    step(ic<0>{}, it);
-    step(ic<1 % NS>{}, it + 1);
-    if (NS > 2) step(ic<2 % NS>{}, it + 2);
-    if (NS > 3) step(ic<3 % NS>{}, it + 3);
+  constexpr int KR = G::KSTEPS < 4 ? G::KSTEPS : 4;
+  // first key and tile addresses of the listed blocks being walked (wave-uniform)
+  int c0C = 0, c0N = 0;
+  uint64_t bvC = 0, bkN = 0, bvN = 0;
+  bool hasN = false;
+  auto position = [&](auto j_c, auto last_c, int h) __attribute__((always_inline)) {
+    constexpr int J = decltype(j_c)::value;  // h % 2
+    constexpr bool LAST = decltype(last_c)::value != 0;  // no tile h+1: only the second half of block A's arithmetic and block B's MFMAs
+    constexpr uint32_t KOFF = (J ^ 1) * TILEB, VOFF = J * TILEB;  // K of tile h+1, V of tile h
+    f32x16& Sc = S[J];
+    f32x16& Sn = S[J ^ 1];
+    uint32_t (&Pc)[8] = Pb[J];
+    uint32_t (&Pn)[8] = Pb[J ^ 1];
+    // Tiles 2q and 2q+1 are the halves of listed block q.  An even position
+    // (h = 2q) looks up block q+1 ("N"); block q ("C") was looked up two
+    // positions ago.  Requests: even h: K of N's first half, V of C's second
+    // half; odd h: K of N's second half, V of N's first half.
+    if constexpr (J == 0) {
+      const int bn = (h >> 1) + 1;
+      hasN = bn < n_blk;
+      if (hasN) {
+        if ((bn >> 6) != col_chunk) {  // walked into the next 64 entries of the list
+          ++col_chunk;
+          col_cur = col_nxt;
+          col_nxt = load_cols(col_chunk + 1);
+        }
+        c0N = __builtin_amdgcn_readlane(col_cur, bn & 63) * kTileN;
+        bkN = kv.k_base + (uint64_t)(uint32_t)c0N * dma.k_pitch;
+        bvN = kv.v_base + (uint64_t)(uint32_t)c0N * dma.v_pitch;
+      }
+    }
+    const bool has1 = J == 0 ? true : hasN, has2 = hasN;
+    const int k0n = J == 0 ? c0C + TN : c0N;  // the tile scored here, whose V is requested here
+    const int k0r = J == 0 ? c0N : c0N + TN;  // the tile whose K is requested here
+    const bool kwhole = k0r + TN <= len, vwhole = k0n + TN <= len;
+    if (!LAST) {
+      if (has2 && !kwhole) dma.template tensor_tile<J, false>(kv, k0r);
+      if (has1 && !vwhole) dma.template tensor_tile<J ^ 1, true>(kv, k0n);
+    }
+    typename DMA::Drip dK, dV;
+    dK.on = DMA::uniform64((has2 && kwhole) ? ~0ull : 0ull);
+    dK.kt = J == 0 ? bkN : bkN + (uint64_t)(TN * dma.k_pitch);
+    dK.sK = dma.lds0 + J * TILEB;
+    dV.on = DMA::uniform64((has1 && vwhole) ? ~0ull : 0ull);
+    dV.vt = J == 0 ? bvC + (uint64_t)(TN * dma.v_pitch) : bvN;
+    dV.sV = dma.lds0 + VBASE + (J ^ 1) * TILEB;
+    dK.vt = 0; dK.sV = 0; dV.kt = 0; dV.sK = 0;
+
+    i32x4 kf[KR], vf[G::NDB];
+    __builtin_amdgcn_s_setprio(3);
+    if (!LAST) {
+#pragma unroll
+      for (int c = 0; c < KR; ++c) kf[c] = fr.load_k(KOFF, 0, c);
+    }
+    // the K fragments were requested a moment ago (their tile was published by
+    // the barrier just passed): the first pair of exponentials goes in front of
+    // the first MFMA, and the last two MFMAs have no arithmetic behind them
+    exp_first(Sc, 4);
+    exp_second(4, Pc, rsv[J]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      if (c < G::KSTEPS && !LAST) {
+        const f32x16 acc = (c == 0) ? (f32x16){0} : Sn;
+        Sn = Elem<T>::mfma(kf[c % KR], Qf[c], acc);
+        if (c + KR < G::KSTEPS) kf[c % KR] = fr.load_k(KOFF, 0, c + KR);
+      }
+      if (c >= 8 - G::NDB) vf[c - (8 - G::NDB)] = fr.load_v(VOFF, 0, c - (8 - G::NDB));
+      if (!LAST) {
+#pragma unroll
+        for (int k = c * 2 * IPW / 8; k < (c + 1) * 2 * IPW / 8; ++k) dma.one((k & 1) ? dV : dK, k);
+      }
+      if (c < 6) {
+        if ((c & 1) == 0)
+          exp_first(Sc, 5 + c / 2);
+        else
+          exp_second(5 + c / 2, Pc, rsv[J]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("" : "+v"(Pc[4]), "+v"(Pc[5]), "+v"(Pc[6]), "+v"(Pc[7]), "+v"(rsv[J]));
+    // a row that has not met a visible key yet has no reference point: exact path
+    if (__builtin_amdgcn_ballot_w64(!(rsv[J] <= kRowSumLimit) || m == -INFINITY) != 0) exact_fix(Sc, Pc, rsv[J]);
+    l += rsv[J];
+    if (!LAST) mask_tile(k0n, Sn);
+    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int sl = 0; sl < 8; ++sl) {
+      if (sl < 2 * G::NDB) {
+        const int kk = sl / G::NDB, db = sl % G::NDB;
+        const i32x4 pf = {(int)Pc[4 * kk], (int)Pc[4 * kk + 1], (int)Pc[4 * kk + 2], (int)Pc[4 * kk + 3]};
+        O[db] = Elem<T>::mfma(vf[db], pf, O[db]);
+        if (kk == 0) vf[db] = fr.load_v(VOFF, 1, db);
+      }
+      if (!LAST) {
+        if ((sl & 1) == 0)
+          exp_first(Sn, sl / 2);
+        else
+          exp_second(sl / 2, Pn, rsv[J ^ 1]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (!LAST) {
+      asm volatile("" : "+v"(Pn[0]), "+v"(Pn[1]), "+v"(Pn[2]), "+v"(Pn[3]), "+v"(rsv[J ^ 1]));
+      // K(h+2) and V(h+1) must have landed and everyone must be done with K(h+1) and V(h)
+      if constexpr (J == 1) {
+        c0C = c0N;
+        bvC = bvN;
+      }
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+      __syncthreads();
+    }
+  };
+
+  if (n_tiles > 0) {
+    c0C = __builtin_amdgcn_readlane(col_cur, 0) * kTileN;
+    bvC = kv.v_base + (uint64_t)(uint32_t)c0C * dma.v_pitch;
+    dma.template tile<0>(kv, c0C);
+    dma.template tensor_tile<1, false>(kv, c0C + TN);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    __syncthreads();
+    {
+      // scores of tile 0, its exact row maximum as the first reference point,
+      // the probabilities of its first 8 keys
+      f32x16 acc = (f32x16){0};
+#pragma unroll
+      for (int c = 0; c < G::KSTEPS; ++c) acc = Elem<T>::mfma(fr.load_k(0u, 0, c), Qf[c], acc);
+      S[0] = acc;
+      mask_tile(c0C, S[0]);
+      exact_fix(S[0], Pb[0], rsv[0]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        exp_first(S[0], i);
+        exp_second(i, Pb[0], rsv[0]);
+      }
+    }
+    __syncthreads();  // position 0 requests K(2) into the stage of K(0), which the other wave may still be reading
+    int h = 0;
+    for (; h + 2 < n_tiles; h += 2) {
+      position(ic<0>{}, ic<0>{}, h);
+      position(ic<1>{}, ic<0>{}, h + 1);
+    }
+    position(ic<0>{}, ic<0>{}, h);
+    position(ic<1>{}, ic<1>{}, h + 1);
+    __builtin_amdgcn_s_setprio(0);
+    __syncthreads();  // every wave is done with the tiles: the staging below reuses them
   }
-  if (it < n_tiles) step(ic<0>{}, it++);
-  if (it < n_tiles) step(ic<1 % NS>{}, it++);
-  if (NS > 3 && it < n_tiles) step(ic<2 % NS>{}, it++);
 
   // ---- epilogue: normalise, transpose through LDS, coalesced 16-byte stores
   const float l_tot = sum_with_other_half(l);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   if (p.lse && fr.lh == 0 && qrow < len) {
-    float* lp = p.lse + g.lse_off + h * p.lse_sh;
+    float* lp = p.lse + g.lse_off + hd * p.lse_sh;
     lp[(int64_t)qrow * p.lse_ss] = l_tot > 0.f ? m + fast_log2(l_tot) : -INFINITY;
   }
   unsigned char* stage = smem + wave * 32 * OROWB;
@@ -950,7 +1043,7 @@ int launch_one(const PrefillParams& p, hipStream_t s) {
   constexpr int TN = SPARSE ? kSparseTileKeys : kTileN;
   void (*kern)(const PrefillParams);
   if constexpr (SPARSE)
-    kern = sparse_kernel<T, D, NW, NS, TN>;
+    kern = sparse_kernel<T, D>;
   else
     kern = dense_kernel<T, D>;
   constexpr size_t lds = prefill_lds_bytes<D, NW, NS, TN>();
