@@ -91,6 +91,35 @@ def test_full_lower_triangle_equals_dense():
     assert (lse - dlse).abs().max().item() <= LSE_TOL
 
 
+def test_listed_blocks_past_the_sequence_end_and_above_the_diagonal():
+    """A mask shared by sequences of different lengths names blocks that lie
+    past the end of the shorter ones, and a full (not lower-triangular) mask
+    names blocks above the diagonal: both are masked per token.  Lengths that
+    are multiples of the block size take the kernel's unmasked-load loop only
+    when every listed block ends inside the sequence."""
+    import tritonops_amd as ta
+
+    Hq, Hkv, D = 4, 2, 128
+    lens = torch.tensor([64, 256, 128, 320, 192], dtype=torch.int32)
+    cu = cu_from(lens)
+    T = int(cu[-1])
+    q, k, v = randn((1, T, Hq, D), 1), randn((1, T, Hkv, D), 2), randn((1, T, Hkv, D), 3)
+    nqb = 5
+    tril = np.tril(np.ones((nqb, nqb), dtype=bool))
+    want, want_lse = orc.block_sparse_attention(q, k, v, cu, tril, faithful=False, return_lse=True)
+    # the lower triangle through the mask form (its lists reach past the shorter sequences)
+    got, lse = ta.flash_attn_sparse_triton(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), block_mask=tril)
+    assert_close(got, want, TOL)
+    assert (lse.cpu() - want_lse).abs().max() <= LSE_TOL
+    # every block listed for every row, as a hand-made CSR (the mask form refuses blocks above the diagonal)
+    row_ptr = torch.arange(0, nqb * nqb + 1, nqb, dtype=torch.int32).cuda()
+    col_idx = torch.arange(nqb, dtype=torch.int32).repeat(nqb).cuda()
+    got, lse = ta.flash_attn_sparse_triton(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), row_ptr=row_ptr, col_idx=col_idx,
+                                           csr_strides=(0, 0, 0, 0))
+    assert_close(got, want, TOL)
+    assert (lse.cpu() - want_lse).abs().max() <= LSE_TOL
+
+
 def test_batched_layout_full_size_mask():
     """Benchmark-shaped mask (256x256 blocks, band 8 + 4 sinks + 10 %) on a
     reduced batch/head count, [B,H,S,D] layout; checked on sampled query blocks

@@ -175,6 +175,16 @@ struct TileDma {
     d.sV = lds0 + VBASE + ST * TILEB;
     return d;
   }
+  // the same for a tile whose loads are all on (no exec mask; not for D = 96,
+  // whose rows have dead chunks)
+  __device__ __forceinline__ void one_on(const Drip& d, int k) const {
+    const int t = k >> 1;
+    const int inst = wave + NW * t;
+    if (k & 1)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff[t]), "s"(d.vt), "s"(d.sV + inst * 1024) : "memory");
+    else
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(koff[t]), "s"(d.kt), "s"(d.sK + inst * 1024) : "memory");
+  }
   __device__ __forceinline__ void one(const Drip& d, int k) const {
     const int t = k >> 1;
     const int inst = wave + NW * t;
@@ -312,6 +322,9 @@ struct TileDma {
 // read with v_readlane: a memory load inside the tile loop would have to be
 // waited for with vmcnt(0), which also drains the tiles requested a moment
 // ago.  A block's two tiles share one list lookup and one address product.
+// When every listed block ends inside the sequence (the usual case: lengths
+// that are multiples of the block size) the walk runs in a copy of the loop
+// whose loads carry no exec mask and that has no path for clamped tiles.
 template <typename T, int D>
 __global__ void __launch_bounds__(kSparseRows * 2) __attribute__((amdgpu_waves_per_eu(2)))
 sparse_kernel(const PrefillParams p) {
@@ -356,6 +369,16 @@ sparse_kernel(const PrefillParams p) {
   };
   int col_chunk = 0;
   int col_cur = load_cols(0), col_nxt = load_cols(1);
+  // does every listed block end inside the sequence?  (A list may name blocks
+  // past the end of a short sequence: their rows are clamped and masked.)
+  bool all_inside;
+  {
+    int mx = max(col_cur, col_nxt);
+    for (int c = 2; c * 64 < n_blk; ++c) mx = max(mx, load_cols(c));
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) mx = max(mx, __shfl_xor(mx, off));
+    all_inside = (__builtin_amdgcn_readfirstlane(mx) + 1) * kTileN <= len;
+  }
   // ---- Q^T operands: lane (query lq, half lh) holds d = 16c + 8lh .. +7
   i32x4 Qf[G::KSTEPS];
   {
@@ -437,8 +460,10 @@ sparse_kernel(const PrefillParams p) {
   int c0C = 0, c0N = 0;
   uint64_t bvC = 0, bkN = 0, bvN = 0;
   bool hasN = false;
-  auto position = [&](auto j_c, auto last_c, int h) __attribute__((always_inline)) {
+  auto position = [&](auto j_c, auto last_c, auto steady_c, int h) __attribute__((always_inline)) {
     constexpr int J = decltype(j_c)::value;  // h % 2
+    // both requested tiles exist and lie inside the sequence: loads without a mask
+    constexpr bool STEADY = decltype(steady_c)::value != 0 && D != 96;
     constexpr bool LAST = decltype(last_c)::value != 0;  // no tile h+1: only the second half of block A's arithmetic and block B's MFMAs
     constexpr uint32_t KOFF = (J ^ 1) * TILEB, VOFF = J * TILEB;  // K of tile h+1, V of tile h
     f32x16& Sc = S[J];
@@ -466,16 +491,21 @@ sparse_kernel(const PrefillParams p) {
     const bool has1 = J == 0 ? true : hasN, has2 = hasN;
     const int k0n = J == 0 ? c0C + TN : c0N;  // the tile scored here, whose V is requested here
     const int k0r = J == 0 ? c0N : c0N + TN;  // the tile whose K is requested here
-    const bool kwhole = k0r + TN <= len, vwhole = k0n + TN <= len;
-    if (!LAST) {
-      if (has2 && !kwhole) dma.template tensor_tile<J, false>(kv, k0r);
-      if (has1 && !vwhole) dma.template tensor_tile<J ^ 1, true>(kv, k0n);
-    }
     typename DMA::Drip dK, dV;
-    dK.on = DMA::uniform64((has2 && kwhole) ? ~0ull : 0ull);
+    dK.on = dV.on = ~0ull;
+    if constexpr (!STEADY) {
+      // a tile that reaches past the sequence end at once (clamped rows), a
+      // whole tile one load at a time behind the MFMAs below
+      const bool kwhole = k0r + TN <= len, vwhole = k0n + TN <= len;
+      if (!LAST) {
+        if (has2 && !kwhole) dma.template tensor_tile<J, false>(kv, k0r);
+        if (has1 && !vwhole) dma.template tensor_tile<J ^ 1, true>(kv, k0n);
+      }
+      dK.on = DMA::uniform64((has2 && kwhole) ? ~0ull : 0ull);
+      dV.on = DMA::uniform64((has1 && vwhole) ? ~0ull : 0ull);
+    }
     dK.kt = J == 0 ? bkN : bkN + (uint64_t)(TN * dma.k_pitch);
     dK.sK = dma.lds0 + J * TILEB;
-    dV.on = DMA::uniform64((has1 && vwhole) ? ~0ull : 0ull);
     dV.vt = J == 0 ? bvC + (uint64_t)(TN * dma.v_pitch) : bvN;
     dV.sV = dma.lds0 + VBASE + (J ^ 1) * TILEB;
     dK.vt = 0; dK.sV = 0; dV.kt = 0; dV.sK = 0;
@@ -502,7 +532,12 @@ sparse_kernel(const PrefillParams p) {
       if (c >= 8 - G::NDB) vf[c - (8 - G::NDB)] = fr.load_v(VOFF, 0, c - (8 - G::NDB));
       if (!LAST) {
 #pragma unroll
-        for (int k = c * 2 * IPW / 8; k < (c + 1) * 2 * IPW / 8; ++k) dma.one((k & 1) ? dV : dK, k);
+        for (int k = c * 2 * IPW / 8; k < (c + 1) * 2 * IPW / 8; ++k) {
+          if constexpr (STEADY)
+            dma.one_on((k & 1) ? dV : dK, k);
+          else
+            dma.one((k & 1) ? dV : dK, k);
+        }
       }
       if (c < 6) {
         if ((c & 1) == 0)
@@ -570,12 +605,20 @@ sparse_kernel(const PrefillParams p) {
     }
     __syncthreads();  // position 0 requests K(2) into the stage of K(0), which the other wave may still be reading
     int h = 0;
-    for (; h + 2 < n_tiles; h += 2) {
-      position(ic<0>{}, ic<0>{}, h);
-      position(ic<1>{}, ic<0>{}, h + 1);
+    if (all_inside) {
+      // every listed block lies inside the sequence: the loop whose loads carry no mask
+      for (; h + 2 < n_tiles; h += 2) {
+        position(ic<0>{}, ic<0>{}, ic<1>{}, h);
+        position(ic<1>{}, ic<0>{}, ic<1>{}, h + 1);
+      }
+    } else {
+      for (; h + 2 < n_tiles; h += 2) {
+        position(ic<0>{}, ic<0>{}, ic<0>{}, h);
+        position(ic<1>{}, ic<0>{}, ic<0>{}, h + 1);
+      }
     }
-    position(ic<0>{}, ic<0>{}, h);
-    position(ic<1>{}, ic<1>{}, h + 1);
+    position(ic<0>{}, ic<0>{}, ic<0>{}, h);
+    position(ic<1>{}, ic<1>{}, ic<0>{}, h + 1);
     __builtin_amdgcn_s_setprio(0);
     __syncthreads();  // every wave is done with the tiles: the staging below reuses them
   }
