@@ -63,3 +63,56 @@ def test_block_sparse_prefill_random_masks(seed):
     want = orc.block_sparse_attention(q, k, v, cu, m)
     got, _ = ta.flash_attn_sparse_triton(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), None, block_mask=m)
     assert _rel(got, want) <= 2e-2, (S, H, Hkv, D, dt)
+
+
+WINDOW_LENGTHS = [1, 31, 33, 64, 65, 127, 128, 192, 200, 257, 320, 384, 513, 700, 1000]
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_window_sparse_prefill_random_windows(seed):
+    """Ragged batches through the window form with windows small enough that a
+    row's first listed tile can lie wholly outside its window (the row then has
+    no reference point for its probabilities yet) and with large scores (the
+    reference point has to move).  Output and LSE against the oracle; rows
+    without any visible key must come back as o = 0, lse = -inf."""
+    import tritonops_amd as ta
+
+    rnd = random.Random(200 + seed)
+    lens = [rnd.choice(WINDOW_LENGTHS) for _ in range(rnd.randint(1, 4))]
+    Hkv = rnd.choice([1, 2, 4])
+    Hq = Hkv * rnd.choice([1, 2, 4])
+    D = rnd.choice([64, 96, 128])
+    dt = rnd.choice([torch.bfloat16, torch.float16])
+    lw = rnd.choice([1, 16, 32, 33, 64, 100, 128, 200, 512])
+    gw = rnd.choice([0, 0, 1, 16, 64, 65, 128, 300])
+    amp = rnd.choice([1.0, 1.0, 4.0, 12.0])
+    cu = cu_from(torch.tensor(lens, dtype=torch.int32))
+    T = int(cu[-1])
+    q = randn((1, T, Hq, D), 1 + seed, dt) * amp
+    k, v = randn((1, T, Hkv, D), 2 + seed, dt), randn((1, T, Hkv, D), 3 + seed, dt)
+    want, want_lse = orc.flash_attn_sparse_torch(q, k, v, cu, None, lw, gw, faithful=False, return_lse=True)
+    got, lse = ta.flash_attn_sparse_triton(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), None, lw, gw)
+    case = (lens, Hq, Hkv, D, dt, lw, gw, amp)
+    assert _rel(got, want) <= 2e-2, case
+    lse = lse.cpu()
+    fin = torch.isfinite(want_lse)
+    assert (torch.isfinite(lse) == fin).all(), case
+    if fin.any():
+        assert (lse[fin] - want_lse[fin]).abs().max().item() <= 2e-2, case
+
+
+def test_block_list_longer_than_the_list_registers():
+    """More than 128 listed blocks per row: the 64-entry list registers are
+    reloaded twice along the walk.  A full lower triangle must give the dense
+    kernel's result."""
+    import tritonops_amd as ta
+
+    S, H, D = 9000, 1, 64
+    nb = (S + 63) // 64
+    m = torch.ones(nb, nb, dtype=torch.bool).tril()
+    cu = cu_from(torch.tensor([S], dtype=torch.int32))
+    q, k, v = (randn((1, S, H, D), s) for s in (5, 6, 7))
+    got, lse = ta.flash_attn_sparse_triton(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), block_mask=m)
+    dense, dlse = ta.flash_attn_triton_fwd(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), D ** -0.5 * ta.LOG2E)
+    assert _rel(got, dense.cpu()) <= 1e-2
+    assert (lse - dlse).abs().max().item() <= 2e-2
