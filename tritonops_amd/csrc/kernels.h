@@ -153,7 +153,9 @@ int launch_xent_dlogits(const XentGradParams& p, int dtype, hipStream_t s);
 // Query rows per workgroup of the two prefill kernels.
 constexpr int kDenseRows = 256;
 constexpr int kSparseRows = 64;
-// LDS stages (KV tiles resident per workgroup) of the two prefill kernels.
+// LDS stages of the two prefill kernels: KV tiles resident per workgroup
+// (dense), K tiles and V tiles resident per workgroup (block-sparse: the K
+// ring runs one tile ahead of the V ring).
 constexpr int kDenseStages = 4;
 constexpr int kSparseStages = 2;
 // Keys per LDS tile of the block-sparse kernel: a 64-key block is walked as two
