@@ -116,3 +116,35 @@ def test_block_list_longer_than_the_list_registers():
     dense, dlse = ta.flash_attn_triton_fwd(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), D ** -0.5 * ta.LOG2E)
     assert _rel(got, dense.cpu()) <= 1e-2
     assert (lse - dlse).abs().max().item() <= 2e-2
+
+
+DENSE_LENGTHS = [0, 1, 2, 31, 33, 64, 65, 128, 129, 192, 255, 256, 257, 300, 384, 385, 511, 513, 640, 769, 1024, 1100]
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_dense_forward_random_ragged_batches(seed):
+    """Up to six sequences per batch, lengths on either side of the 64-key tile
+    and the 256-row work item, so that consecutive work items of a workgroup
+    have zero to five tiles (the requests of the next item's tiles are counted
+    against the output stores of the one before)."""
+    import tritonops_amd as ta
+
+    rnd = random.Random(300 + seed)
+    lens = [rnd.choice(DENSE_LENGTHS) for _ in range(rnd.randint(1, 6))]
+    if sum(lens) == 0:
+        lens[0] = 5
+    Hkv = rnd.choice([1, 2, 4])
+    Hq = Hkv * rnd.choice([1, 2, 4])
+    D = rnd.choice([64, 96, 128])
+    dt = rnd.choice([torch.bfloat16, torch.float16])
+    amp = rnd.choice([1.0, 1.0, 5.0])
+    cu = cu_from(torch.tensor(lens, dtype=torch.int32))
+    T = int(cu[-1])
+    q = randn((1, T, Hq, D), 1 + seed, dt) * amp
+    k, v = randn((1, T, Hkv, D), 2 + seed, dt), randn((1, T, Hkv, D), 3 + seed, dt)
+    want, want_lse = orc.varlen_masked_attention(q, k, v, cu, orc.causal_mask, None, False, True)
+    got, lse = ta.flash_attn_triton_fwd(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), D ** -0.5 * ta.LOG2E)
+    case = (lens, Hq, Hkv, D, dt, amp)
+    assert _rel(got, want) <= 2e-2, case
+    fin = torch.isfinite(want_lse)
+    assert (lse.cpu()[fin] - want_lse[fin]).abs().max().item() <= 2e-2, case
