@@ -570,6 +570,207 @@ def run_fused_xent(steps, warmup):
     }
 
 
+def _packed_fwd_args(q, k, v, o, lse, cu, max_len, causal=True):
+    """mi_attn_fwd_args for packed [1,T,H,D] tensors with cu_seqlens."""
+    from tritonops_amd import _lib
+    a = _lib.AttnFwdArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _lib.MI_DTYPE_BF16
+    a.q, a.k, a.v, a.o, a.lse = (t.data_ptr() for t in (q, k, v, o, lse))
+    for n, t in (("q", q), ("k", k), ("v", v), ("o", o)):
+        setattr(a, n + "_stride_s", t.stride(1))
+        setattr(a, n + "_stride_h", t.stride(2))
+    a.lse_stride_s, a.lse_stride_h = lse.stride(1), lse.stride(2)
+    a.cu_seqlens = cu.data_ptr()
+    a.batch, a.heads_q, a.heads_kv, a.max_seqlen, a.head_dim = cu.numel() - 1, q.shape[2], k.shape[2], max_len, q.shape[3]
+    a.causal = 1 if causal else 0
+    a.scale_log2 = q.shape[3] ** -0.5 * LOG2E
+    a.total_rows = q.shape[1]
+    return a
+
+
+def run_dense_packed(steps, warmup):
+    """The reference's own call form of the dense forward: packed [1,T,H,D] tensors + cu_seq_lens through
+    flash_attention(q, k, v, cu) (= flash_attn_triton.apply, flash_attn_triton.py:816-846), at the headline size
+    (4 sequences of 8192 tokens) and on a ragged mix of the same 32768 tokens."""
+    import tritonops_amd as ta
+    T, H, D = 32768, 32, 128
+    q, k, v = (_randn((1, T, H, D), s) for s in (0, 1, 2))
+    mixes = {"4x8192": [8192] * 4, "ragged": [8192, 4096, 12288, 2048, 1024, 5120]}
+    out = {}
+    for name, lens in mixes.items():
+        cu = torch.zeros(len(lens) + 1, dtype=torch.int32)
+        cu[1:] = torch.cumsum(torch.tensor(lens), 0)
+        cu = cu.cuda()
+        fn = lambda: ta.flash_attention(q, k, v, cu, return_lse=True)
+        ms = _time_steps(fn, steps, warmup)
+        o, lse = fn()
+        o2, lse2 = torch.empty_like(o), torch.empty_like(lse)
+        kms = _event_ms(0, _packed_fwd_args(q, k, v, o2, lse2, cu, max(lens)), steps, warmup)
+        flop = sum(2.0 * H * n * (n + 1) * D for n in lens)
+        # parity on the benchmark tensors: two heads x three 64-row blocks of the first, a middle and the last sequence
+        err = err_lse = 0.0
+        for si in (0, len(lens) // 2, len(lens) - 1):
+            s0, n = int(cu[si]), lens[si]
+            keys = torch.arange(n, device="cuda")
+            for h in (0, 21):
+                for r0 in (0, n // 2, n - 64):
+                    rows = torch.arange(r0, r0 + 64, device="cuda")
+                    want, want_lse = _ref_rows(q[0, s0:s0 + n, h], k[0, s0:s0 + n, h], v[0, s0:s0 + n, h], rows,
+                                               D ** -0.5, keys[None, :] <= rows[:, None])
+                    err = max(err, _err(o[0, s0 + rows, h], want))
+                    err_lse = max(err_lse, _err(lse[0, s0 + rows, h], want_lse))
+        out[name] = dict(ms=ms, kms=kms, flop=flop, err=err, err_lse=err_lse)
+    m = out["4x8192"]
+    r = out["ragged"]
+    return {
+        "name": "dense_causal_packed", "ms_per_step": m["ms"], "kernel_ms": m["kms"],
+        "metric": "attn_fwd_tflops", "unit": "TFLOP/s", "value": m["flop"] / (m["ms"] * 1e-3) / 1e12,
+        "max_abs_err": max(m["err"], r["err"]), "max_abs_err_lse2": max(m["err_lse"], r["err_lse"]),
+        "err_sample": "o and lse of 2 heads x 3 blocks of 64 query rows in 3 sequences of each mix against fp32 torch math on the device",
+        "roofline": {"bound": "mfma", "achieved": m["flop"] / (m["kms"] * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "kernel": KERNELS["dense_causal"]},
+        "config": {"workload": "dense causal fwd bf16, packed [1,32768,32,128] + cu_seq_lens for 4 x 8192 tokens, through "
+                               "flash_attention(q, k, v, cu_seq_lens) with uninitialised outputs (the library zeroes "
+                               "rows outside the sequences) and the longest length cached per cu_seq_lens tensor",
+                   "flop_per_step": m["flop"],
+                   "wall_over_kernel": m["ms"] / m["kms"],
+                   "ragged_mix": {"lens": mixes["ragged"], "ms_per_step": r["ms"], "kernel_ms": r["kms"],
+                                  "flop_per_step": r["flop"], "tflops": r["flop"] / (r["kms"] * 1e-3) / 1e12,
+                                  "frac": r["flop"] / (r["kms"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                                  "wall_over_kernel": r["ms"] / r["kms"]}},
+    }
+
+
+def _window_pairs(n, lw, gw):
+    """Allowed (q, k) pairs of one sequence of n tokens under k <= q and (q - k < lw or k < gw)."""
+    import numpy as np
+    qi = np.arange(n, dtype=np.int64)
+    return int((np.minimum(qi + 1, lw) + np.maximum(0, np.minimum(gw, qi + 1 - lw))).sum())
+
+
+def run_window_sparse_prefill(steps, warmup):
+    """The reference's own sparse prefill form: token windows on packed tensors
+    (flash_attn_sparse_attn_triton.py:237-326), local window 1024, global window 128, 4 sequences of 8192 tokens."""
+    import tritonops_amd as ta
+    from tritonops_amd import _lib, masks
+    B, H, S, D, LW, GW = 4, 16, 8192, 128, 1024, 128
+    T = B * S
+    q, k, v = (_randn((1, T, H, D), s) for s in (0, 1, 2))
+    cu = (torch.arange(B + 1, dtype=torch.int32) * S).cuda()
+    fn = lambda: ta.flash_attn_sparse_triton(q, k, v, cu, None, LW, GW)
+    ms = _time_steps(fn, steps, warmup)
+    o, lse = fn()
+    row_ptr, col_idx, strides = masks.window_csr(S // 64, LW, GW, "cuda")
+    o2, lse2 = torch.empty_like(o), torch.empty_like(lse)
+    a = _lib.AttnSparseArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _lib.MI_DTYPE_BF16
+    a.q, a.k, a.v, a.o, a.lse = (t.data_ptr() for t in (q, k, v, o2, lse2))
+    for n, t in (("q", q), ("k", k), ("v", v), ("o", o2)):
+        setattr(a, n + "_stride_s", t.stride(1))
+        setattr(a, n + "_stride_h", t.stride(2))
+    a.lse_stride_s, a.lse_stride_h = lse2.stride(1), lse2.stride(2)
+    a.cu_seqlens = cu.data_ptr()
+    a.row_ptr, a.col_idx = row_ptr.data_ptr(), col_idx.data_ptr()
+    a.row_ptr_stride_b, a.row_ptr_stride_h, a.col_idx_stride_b, a.col_idx_stride_h = strides
+    a.batch, a.heads_q, a.heads_kv, a.max_seqlen, a.head_dim = B, H, H, S, D
+    a.block_size, a.window_local, a.window_global = 64, LW, GW
+    a.scale_log2 = D ** -0.5 * LOG2E
+    a.total_rows = T
+    kms = _event_ms(1, a, steps, warmup)
+    flop = 4.0 * D * _window_pairs(S, LW, GW) * H * B
+    err = err_lse = 0.0
+    keys = torch.arange(S, device="cuda")
+    for b in (0, 3):
+        for r0 in (0, 1024, 4160, S - 64):
+            rows = torch.arange(r0, r0 + 64, device="cuda")
+            allow = (keys[None, :] <= rows[:, None]) & ((rows[:, None] - keys[None, :] < LW) | (keys[None, :] < GW))
+            sl = slice(b * S, (b + 1) * S)
+            want, want_lse = _ref_rows(q[0, sl].transpose(0, 1), k[0, sl].transpose(0, 1), v[0, sl].transpose(0, 1),
+                                       rows, D ** -0.5, allow)
+            err = max(err, _err(o[0, b * S + rows].transpose(0, 1), want))
+            err_lse = max(err_lse, _err(lse[0, b * S + rows].transpose(0, 1), want_lse))
+    return {
+        "name": "window_sparse_prefill", "ms_per_step": ms, "kernel_ms": kms,
+        "metric": "sparse_attn_fwd_tflops", "unit": "TFLOP/s", "value": flop / (ms * 1e-3) / 1e12,
+        "max_abs_err": err, "max_abs_err_lse2": err_lse,
+        "err_sample": "o and lse of all heads x 4 blocks of 64 query rows in 2 of the 4 sequences against masked fp32 torch math on the device",
+        "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "kernel": KERNELS["block_sparse"]},
+        "config": {"workload": "window-sparse causal fwd bf16, packed [1,32768,16,128] + cu_seqlens for 4 x 8192 tokens, local "
+                               "window 1024, global window 128, through flash_attn_sparse_triton(q, k, v, cu, None, 1024, 128)",
+                   "flop_per_step": flop, "wall_over_kernel": ms / kms,
+                   "note": "FLOP counts the allowed (q, k) pairs only; the kernel walks whole 64x64 blocks that hold one"},
+    }
+
+
+def run_window_sparse_decode(steps, warmup):
+    """The reference's own sparse decoding form: flash_attention_sparse_decoding(q, k, v, cu_seq_lens, 256, 4096)
+    (flash_attn_decoding_sparse.py:222-365) at the KV size of the block-list configuration."""
+    import tritonops_amd as ta
+    from tritonops_amd import _lib
+    B, Hq, Hkv, L, D, GW, LW = 32, 32, 8, 131072, 128, 256, 4096
+    g = torch.Generator().manual_seed(1)
+    lens = (L - torch.randint(0, 64, (B,), generator=g)).to(torch.int32)
+    cu = torch.zeros(B + 1, dtype=torch.int32)
+    cu[1:] = torch.cumsum(lens, 0)
+    cu_d, lens_d = cu.cuda(), lens.cuda()
+    q = _randn((B, Hq, D), 0)
+    kc, vc = _randn((B, Hkv, L, D), 1), _randn((B, Hkv, L, D), 2)
+    k, v = kc.transpose(1, 2), vc.transpose(1, 2)
+    fn = lambda: ta.flash_attention_sparse_decoding(q, k, v, cu_d, GW, LW)
+    ms = _time_steps(fn, steps, warmup)
+    got = fn()
+    lib = _lib.load()
+    o = torch.empty((B, Hq, D), device="cuda", dtype=torch.bfloat16)
+    a = _lib.DecodeArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _lib.MI_DTYPE_BF16
+    a.q, a.k, a.v, a.o, a.lse = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), None
+    a.q_stride_b, a.q_stride_h = q.stride(0), q.stride(1)
+    a.k_stride_b, a.k_stride_s, a.k_stride_h = k.stride(0), k.stride(1), k.stride(2)
+    a.v_stride_b, a.v_stride_s, a.v_stride_h = v.stride(0), v.stride(1), v.stride(2)
+    a.o_stride_b, a.o_stride_h = o.stride(0), o.stride(1)
+    a.seq_lens, a.cu_seqlens = None, cu_d.data_ptr()
+    a.batch, a.heads_q, a.heads_kv, a.max_seqlen, a.head_dim = B, Hq, Hkv, L, D
+    a.scale_log2 = D ** -0.5 * LOG2E
+    a.split_tokens = 64
+    a.window_form, a.window_local, a.window_global = 1, LW, GW
+    a.max_blocks, a.block_size = GW // 64 + (LW + 63) // 64 + 1, 64
+    a.split_blocks = lib.mi_decode_choose_split_blocks(B, Hkv, a.max_blocks, lib.mi_device_cu_count())
+    nb = lib.mi_decode_workspace_bytes(C.byref(a))
+    ws = torch.empty(nb, device="cuda", dtype=torch.uint8)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), nb
+    k_split = _event_ms(3, a, steps, warmup)
+    k_both = _event_ms(2, a, steps, warmup)
+    nbytes_alg = float(B * Hkv * (GW + LW) * D * 2 * 2)
+    err = 0.0
+    for b in (0, 15, 31):
+        n = int(lens[b])
+        tok = torch.cat([torch.arange(GW), torch.arange(n - LW, n)]).cuda()
+        kk, vv = kc[b][:, tok].float(), vc[b][:, tok].float()
+        sc = torch.einsum("gid,gld->gil", q[b].view(Hkv, Hq // Hkv, D).float(), kk) * D ** -0.5
+        want = torch.einsum("gil,gld->gid", torch.softmax(sc, -1), vv).reshape(Hq, D)
+        err = max(err, _err(got[b], want))
+    return {
+        "name": "window_sparse_decode", "ms_per_step": ms, "kernel_ms": k_both, "splitkv_kernel_ms": k_split,
+        "metric": "sparse_decode_hbm_gbs", "unit": "GB/s", "value": nbytes_alg / (ms * 1e-3) / 1e9,
+        "max_abs_err": err,
+        "err_sample": "3 of the 32 sequences (all heads) against fp32 torch math over the attended tokens on the device",
+        "roofline": {"bound": "hbm", "achieved": nbytes_alg / (k_split * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "kernel": KERNELS["sparse_decode"]},
+        "config": {"workload": "window-sparse decode bf16 B=32 Hq=32 Hkv=8 KV=131072 D=128, global window 256 + local window "
+                               "4096, through flash_attention_sparse_decoding(q, k, v, cu_seq_lens, 256, 4096): two "
+                               "launches, the block list is derived inside the kernel",
+                   "bytes_per_step": nbytes_alg, "split_blocks": int(a.split_blocks),
+                   "wall_over_kernel": ms / k_both,
+                   "note": "kernel_ms is both launches (split-KV + merge), which is what one call costs on the device; "
+                           "the roofline figure is the split-KV launch alone. 0.58 GB per step is little work for 256 "
+                           "CUs: the launch is latency-bound, not bandwidth-bound"},
+    }
+
+
 WORKLOADS = {
     "dense_causal": run_dense_causal,
     "c1_dense_noncausal_small": run_c1_small,
@@ -579,7 +780,33 @@ WORKLOADS = {
     "dense_causal_bwd": run_dense_bwd,
     "rmsnorm": run_rmsnorm,
     "fused_xent": run_fused_xent,
+    "dense_causal_packed": run_dense_packed,
+    "window_sparse_prefill": run_window_sparse_prefill,
+    "window_sparse_decode": run_window_sparse_decode,
 }
+
+# Parity bars: the largest error a workload's own check may report (its figure under "max_abs_err",
+# plus the named extra ones).  A run that exceeds one, or reports a value that is not finite, prints its
+# line with "parity_ok": false and exits with status 1, so that no timing is recorded for a wrong result.
+PARITY_BARS = {
+    "dense_causal": {"max_abs_err": 2e-2, "max_abs_err_lse2": 2e-3},
+    "c1_dense_noncausal_small": {"max_abs_err": 2e-2},
+    "gqa_decode": {"max_abs_err": 2e-2},
+    "block_sparse": {"max_abs_err": 2e-2, "max_abs_err_lse2": 2e-3},
+    "sparse_decode": {"max_abs_err": 2e-2},
+    "dense_causal_bwd": {"max_abs_err": 3e-2},
+    "rmsnorm": {"max_abs_err": 4e-2, "max_rel_err_dw": 1e-2},
+    "fused_xent": {"max_abs_err": 2e-2},
+    "dense_causal_packed": {"max_abs_err": 2e-2, "max_abs_err_lse2": 2e-3},
+    "window_sparse_prefill": {"max_abs_err": 2e-2, "max_abs_err_lse2": 2e-3},
+    "window_sparse_decode": {"max_abs_err": 2e-2},
+}
+
+
+def _parity(r):
+    bars = PARITY_BARS[r["name"]]
+    ok = all(k in r and math.isfinite(r[k]) and r[k] <= bar for k, bar in bars.items())
+    return ok, bars
 
 
 # ----------------------------------------------------------------------------
@@ -687,6 +914,39 @@ def cpu_baseline(name):
                           "(common/rms.py math) on [4096, 4096] bf16 (1/8 of the rows), median of 3; same "
                           "algorithmic-byte formula as the GPU figure",
                 "seconds": t}
+    if name == "dense_causal_packed":
+        S, H, D = 8192, 4, 128
+        q, k, v = (torch.randn((1, S, H, D), generator=g).to(torch.bfloat16) for _ in range(3))
+        cu = torch.tensor([0, S], dtype=torch.int32)
+        t = med(lambda: orc.flash_attn_torch(q, k, v, cu), reps=1)
+        flop = 2.0 * H * S * (S + 1) * D
+        return {"value": flop / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "sample": "torch-CPU var-len causal oracle (flash_attn_triton.py:877-915 math) on one packed sequence of 8192 "
+                          "tokens, 4 of the 32 heads (1/32 of the workload), one timed run after a warm-up; same "
+                          "algorithmic-FLOP formula as the GPU figure",
+                "seconds": t}
+    if name == "window_sparse_prefill":
+        S, H, D, LW, GW = 8192, 4, 128, 1024, 128
+        q, k, v = (torch.randn((1, S, H, D), generator=g).to(torch.bfloat16) for _ in range(3))
+        cu = torch.tensor([0, S], dtype=torch.int32)
+        t = med(lambda: orc.flash_attn_sparse_torch(q, k, v, cu, None, LW, GW), reps=1)
+        flop = 4.0 * D * _window_pairs(S, LW, GW) * H
+        return {"value": flop / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "sample": "torch-CPU window oracle (flash_attn_sparse_attn_triton.py:391-442: full S x S scores, then the "
+                          "mask) on one sequence of 8192 tokens, 4 of the 16 heads (1/16 of the workload), one timed run "
+                          "after a warm-up; same algorithmic-FLOP formula as the GPU figure (allowed pairs only)",
+                "seconds": t}
+    if name == "window_sparse_decode":
+        B, Hq, Hkv, L, D, GW, LW = 1, 32, 8, 131072, 128, 256, 4096
+        lens = (L - torch.randint(0, 64, (B,), generator=g)).to(torch.int32)
+        q = torch.randn((B, Hq, D), generator=g).to(torch.bfloat16)
+        k, v = (torch.randn((B, L, Hkv, D), generator=g, dtype=torch.bfloat16) for _ in range(2))
+        t = med(lambda: orc.flash_attn_sparse_decoding_torch(q, k, v, lens, GW, LW))
+        nb = float(B * Hkv * (GW + LW) * D * 2 * 2)
+        return {"value": nb / t / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+                "sample": "torch-CPU window decode oracle (flash_attn_decoding_sparse.py:368-406) on one of the 32 "
+                          "sequences, median of 3; same algorithmic-byte formula as the GPU figure",
+                "seconds": t}
     if name == "fused_xent":
         from oracle import xent_oracle as xo
         T, D, N = 128, 4096, 128256
@@ -747,6 +1007,7 @@ def main():
         rf["traffic"] = t.get("hbm_bytes_per_launch") if fresh else None
         rf["traffic_source"] = ("profiles/hbm_traffic.json, measured at commit %s" % traffic.get("_commit", "?")
                                 if fresh else "no counter run of this kernel on file")
+        r["parity_ok"], r["parity_bars"] = _parity(r)
         results.append(r)
         torch.cuda.empty_cache()
     head = results[0]
@@ -757,6 +1018,7 @@ def main():
         "dtype": "bf16", "data": "synthetic N(0,1) inputs drawn from a seed, resident in HBM",
         "config": head["config"], "roofline": head["roofline"], "kernel_ms": head["kernel_ms"],
         "max_abs_err": head.get("max_abs_err"), "err_sample": head.get("err_sample"),
+        "parity_ok": all(r["parity_ok"] for r in results), "parity_bars": head["parity_bars"],
         "device": torch.cuda.get_device_name(0),
         "compute_units": torch.cuda.get_device_properties(0).multi_processor_count,
     }
@@ -767,7 +1029,8 @@ def main():
     if len(results) > 1:
         out["other_workloads"] = [
             {k: r[k] for k in ("name", "metric", "value", "unit", "ms_per_step", "kernel_ms", "max_abs_err",
-                               "err_sample", "roofline", "config") if k in r}
+                               "max_abs_err_lse2", "max_rel_err_dw", "err_sample", "parity_ok", "parity_bars",
+                               "roofline", "config") if k in r}
             for r in results[1:]]
         if not a.no_cpu_baseline:
             for r in out["other_workloads"]:
@@ -775,6 +1038,9 @@ def main():
                 if cb is not None:
                     r["cpu_baseline"] = cb
     print(json.dumps(out))
+    if not out["parity_ok"]:
+        bad = [r["name"] for r in results if not r["parity_ok"]]
+        sys.exit("bench.py: parity bar exceeded by %s; the timings above are of wrong results" % ", ".join(bad))
 
 
 if __name__ == "__main__":

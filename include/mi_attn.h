@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define MI_ATTN_ABI_VERSION 5
+#define MI_ATTN_ABI_VERSION 6
 
 /* KV tile edge (tokens) of the prefill kernels and block edge of the block
  * sparse layouts; fixed at build time. */
@@ -78,7 +78,16 @@ typedef enum mi_status {
  *                        cu_seqlens[b]+t; *_stride_b is ignored.
  *   cu_seqlens == NULL : batched. Every sequence has max_seqlen tokens and
  *                        sequence b starts at b * *_stride_b.
- * Rows whose sequence has length 0 are never written.
+ * Rows whose sequence has length 0 are never written.  In the packed form
+ * max_seqlen must bound every length: a longer sequence is cut at max_seqlen
+ * (its later rows are neither read nor written).
+ * total_rows (packed form only): the reference launcher zero-fills o and lse
+ * before its kernel runs (flash_attn_triton.py:608-609), so rows that belong to
+ * no sequence come back as zeros.  With total_rows > 0 the call does the same
+ * for exactly those rows - rows of [0, total_rows) that lie behind
+ * cu_seqlens[batch], or behind the first max_seqlen tokens of their sequence -
+ * with one small extra launch, so the caller can hand in uninitialised
+ * outputs.  0 leaves such rows untouched.
  */
 typedef struct mi_attn_fwd_args {
   uint32_t struct_size;
@@ -97,6 +106,7 @@ typedef struct mi_attn_fwd_args {
   int32_t head_dim;              /* 64, 96 or 128 (q, k and v alike)           */
   int32_t causal;                /* 0 / 1                                      */
   float scale_log2;              /* softmax scale * log2(e), > 0               */
+  int32_t total_rows;            /* packed: rows of o / lse to cover, or 0     */
 } mi_attn_fwd_args;
 
 int mi_attn_fwd(const mi_attn_fwd_args *args, void *stream);
@@ -110,6 +120,8 @@ int mi_attn_fwd(const mi_attn_fwd_args *args, void *stream);
  * summed inside the kernel).  Addressing modes, causal flag and scale as in
  * mi_attn_fwd.  The workspace holds
  * Delta = rowsum(o * dout) in fp32.  Two launches on `stream`.
+ * total_rows as in mi_attn_fwd: with a value > 0 (packed form) the rows of dq,
+ * dk and dv that belong to no sequence are zero-filled by one more launch.
  */
 typedef struct mi_attn_bwd_args {
   uint32_t struct_size;
@@ -134,6 +146,7 @@ typedef struct mi_attn_bwd_args {
   float scale_log2;                  /* the value the forward pass was given   */
   void *workspace;                   /* device, mi_attn_bwd_workspace_bytes()  */
   size_t workspace_bytes;
+  int32_t total_rows;                /* packed: rows of dq/dk/dv to cover, or 0 */
 } mi_attn_bwd_args;
 
 size_t mi_attn_bwd_workspace_bytes(const mi_attn_bwd_args *args);
@@ -160,6 +173,8 @@ int mi_attn_bwd(const mi_attn_bwd_args *args, void *stream);
  *   allowed(q,k) = k <= q and (q - k < window_local or k < window_global).
  * Pass -1 / -1 for a pure block mask.
  * A query row with no allowed key yields o = 0 and lse = -inf.
+ * total_rows as in mi_attn_fwd (the reference launcher zero-fills both outputs,
+ * flash_attn_sparse_attn_triton.py:274-275).
  */
 typedef struct mi_attn_sparse_args {
   uint32_t struct_size;
@@ -184,6 +199,7 @@ typedef struct mi_attn_sparse_args {
   int32_t window_local;          /* tokens, or -1                              */
   int32_t window_global;         /* tokens, or -1                              */
   float scale_log2;
+  int32_t total_rows;            /* packed: rows of o / lse to cover, or 0     */
 } mi_attn_sparse_args;
 
 int mi_attn_fwd_blocksparse(const mi_attn_sparse_args *args, void *stream);
@@ -198,8 +214,10 @@ int mi_attn_fwd_blocksparse(const mi_attn_sparse_args *args, void *stream);
  * q [batch, heads_q, head_dim]; k, v padded per sequence: token t of sequence
  * b, kv-head h at  b*stride_b + t*stride_s + h*stride_h ; only the first
  * seq_lens[b] tokens are read (flash_attn_decoding.py:46-48,80).  The G =
- * heads_q/heads_kv query heads of one kv-head are processed together so every
- * K/V byte is fetched from HBM once.
+ * heads_q/heads_kv query heads of one kv-head are processed together, 32 to a
+ * wavefront, so every K/V byte is fetched once per 32 query heads (the
+ * reference fetches it once per query head, flash_attn_decoding.py:42-45,
+ * 264-268); any ratio G is accepted.
  *
  * Pass 1 splits each sequence into chunks of `split_tokens` tokens (dense) or
  * `split_blocks` listed blocks (sparse); one workgroup per (chunk, kv-head,
@@ -218,6 +236,16 @@ int mi_attn_fwd_blocksparse(const mi_attn_sparse_args *args, void *stream);
  * list an optional token window reproduces flash_attn_decoding_sparse.py
  * :391-396:  allowed(k) = k < window_global or k >= seq_len - window_local
  * (pass -1/-1 to disable).
+ *
+ * Window form (window_form = 1, block_idx ignored): the list is not read from
+ * memory but derived per sequence from (seq_len, window_global, window_local),
+ * which is all the reference's sparse decoder attends (flash_attn_decoding_
+ * sparse.py:391-396): the blocks of the first window_global tokens, then the
+ * blocks from token max(seq_len - window_local, 0) to the last one, each once,
+ * with the token window applied inside them.  max_blocks must be at least
+ *   ceil(window_global / 64) + ceil(window_local / 64) + 1
+ * (it sizes the chunks and the workspace); block_cnt and include_last_block
+ * are ignored.
  */
 /* Where token t of sequence b lives in k / v (element strides as given):
  *   MI_KV_BATCHED  k + b*k_stride_b + t*k_stride_s            ([batch, max_seqlen, heads_kv, D] view; the
@@ -271,6 +299,7 @@ typedef struct mi_decode_args {
   const int32_t *page_table;     /* paged: device; physical page of logical    */
                                  /* page p of sequence b at [b*stride_b + p]   */
   int64_t page_table_stride_b;
+  int32_t window_form;           /* 1: block list derived from the two windows */
 } mi_decode_args;
 
 /* Number of pass-1 chunks per sequence for these arguments (host only). */
@@ -307,7 +336,10 @@ int mi_decode(const mi_decode_args *args, void *stream);
  * memory, one per GPU, from load time until the process ends.  A call whose
  * mi_decode_workspace_bytes() exceeds that size fails with MI_ERR_WORKSPACE
  * before anything is launched (pick larger split_tokens / split_blocks).
- * The call allocates and frees nothing and records only kernel launches.
+ * The call allocates and frees nothing and records only kernel launches; the
+ * FIRST call on a device also asks the runtime for the buffer's device address
+ * (hipGetSymbolAddress, which may load the code object), so make one call per
+ * device outside capture before recording it into a graph.
  * Every call on one GPU uses the same buffer: calls that overlap on one GPU
  * (different streams, or graphs replayed concurrently) race; serialise them.
  * The buffer keeps the previous call's partials; nothing in it needs to start

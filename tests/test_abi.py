@@ -27,7 +27,7 @@ def test_every_declared_symbol_is_exported(lib):
     assert declared == set(_lib.EXPORTS), "ctypes table and header disagree: %s" % (declared ^ set(_lib.EXPORTS))
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.mi_abi_version() == _lib.MI_ATTN_ABI_VERSION == 5
+    assert lib.mi_abi_version() == _lib.MI_ATTN_ABI_VERSION == 6
 
 
 def test_struct_layout_matches_the_c_compiler(tmp_path):
@@ -91,6 +91,8 @@ def test_fwd_validation(lib):
         (lambda a: setattr(a, "k", 0x1004), "MI_ERR_ALIGNMENT"),
         (lambda a: setattr(a, "v_stride_s", 100), "MI_ERR_STRIDE"),
         (lambda a: setattr(a, "o_stride_b", 4), "MI_ERR_STRIDE"),
+        (lambda a: setattr(a, "total_rows", -1), "MI_ERR_SHAPE"),
+        (lambda a: setattr(a, "total_rows", 64), "MI_ERR_SHAPE"),       # batched form: there are no rows outside the sequences
     ]
     for mutate, want in cases:
         a = _good_fwd()
@@ -105,6 +107,7 @@ def test_fwd_validation(lib):
     a = _good_fwd()
     a.cu_seqlens = 0x2000
     a.o_stride_b = 4
+    a.total_rows = 4096
     assert lib.mi_attn_fwd_validate(C.byref(a)) == 0
 
 
@@ -166,7 +169,8 @@ def test_decode_geometry_and_validation(lib):
         (lambda a: setattr(a, "cu_seqlens", 0x2000), "MI_ERR_NULL_POINTER"),     # both given
         (lambda a: setattr(a, "seq_lens", None), "MI_ERR_NULL_POINTER"),         # none given
         (lambda a: setattr(a, "heads_kv", 0), "MI_ERR_GQA"),
-        (lambda a: (setattr(a, "heads_q", 66), setattr(a, "heads_kv", 2)), "MI_ERR_GQA"),   # 33 per kv head
+        (lambda a: (setattr(a, "heads_q", 66), setattr(a, "heads_kv", 4)), "MI_ERR_GQA"),   # not a multiple
+        (lambda a: setattr(a, "window_form", 2), "MI_ERR_SPARSE_LAYOUT"),
         (lambda a: setattr(a, "k_stride_s", 12), "MI_ERR_STRIDE"),
         # a tile is addressed with 32-bit byte offsets: negative or huge row strides would wrap
         (lambda a: setattr(a, "k_stride_s", -128), "MI_ERR_STRIDE"),
@@ -181,6 +185,24 @@ def test_decode_geometry_and_validation(lib):
     a = _good_decode()
     a.k_stride_s = a.v_stride_s = (1 << 24) - 8
     assert lib.mi_decode_validate(C.byref(a)) == 0
+    # a GQA group of more than 32 query heads is walked in slices of 32
+    a = _good_decode()
+    a.heads_q, a.heads_kv = 66, 2
+    assert lib.mi_decode_validate(C.byref(a)) == 0
+    assert lib.mi_decode_workspace_bytes(C.byref(a)) == 4 * 66 * 8 * 129 * 4
+    # window form: the list is derived in the kernel, block_idx may be NULL
+    a = _good_decode()
+    a.window_form, a.block_size, a.split_blocks = 1, 64, 4
+    a.window_global, a.window_local = 256, 1000
+    a.max_blocks = 4 + 16 + 1
+    assert lib.mi_decode_validate(C.byref(a)) == 0 and lib.mi_decode_num_splits(C.byref(a)) == 6
+    a.include_last_block = 1     # ignored in the window form
+    assert lib.mi_decode_num_splits(C.byref(a)) == 6
+    for mutate in (lambda a: setattr(a, "max_blocks", 20), lambda a: setattr(a, "window_local", -1),
+                   lambda a: setattr(a, "split_blocks", 0), lambda a: setattr(a, "block_size", 32)):
+        b = _lib.DecodeArgs.from_buffer_copy(a)
+        mutate(b)
+        assert lib.mi_status_name(lib.mi_decode_validate(C.byref(b))).decode() == "MI_ERR_SPARSE_LAYOUT", _err(lib)
     # sparse form
     a = _good_decode()
     a.block_idx = 0x5000
@@ -364,9 +386,11 @@ def test_split_blocks_heuristic(lib):
 
 def test_time_launches_rejects_bad_arguments(lib):
     ms = C.c_float()
-    assert lib.mi_time_launches(0, None, 1, 0, None, 0, 1, C.byref(ms)) == -6
+    assert lib.mi_time_launches(0, None, 1, 0, None, 0, 1, C.byref(ms)) == -1
+    assert "non-NULL" in _err(lib)
     a = _good_fwd()
     assert lib.mi_time_launches(12, C.cast(C.byref(a), C.c_void_p), 1, 0, None, 0, 1, C.byref(ms)) == -6
+    assert "kind" in _err(lib)
     assert lib.mi_time_launches(0, C.cast(C.byref(a), C.c_void_p), 0, 0, None, 0, 1, C.byref(ms)) == -6
     a.head_dim = 5
     assert lib.mi_time_launches(0, C.cast(C.byref(a), C.c_void_p), 1, 0, None, 1, 1, C.byref(ms)) == -4

@@ -107,3 +107,54 @@ def test_noalloc_block_list_form_and_size_limit():
     big.batch, big.max_seqlen = 4096, 1 << 20
     rc = lib.mi_decode_noalloc(C.byref(big), None)
     assert lib.mi_status_name(rc).decode() == "MI_ERR_WORKSPACE"
+
+
+def test_noalloc_decode_recorded_into_a_graph_replays_like_mi_decode():
+    """The callers the entry point is for include code under HIP graph
+    capture.  After one call outside capture (which looks up the device address
+    of the static buffer) a captured call records two kernel launches; every
+    replay, over changed inputs and lengths, equals mi_decode bit for bit."""
+    from tritonops_amd import _lib
+
+    lib = _lib.load()
+    B, Hq, Hkv, L, D = 4, 16, 4, 3000, 128
+    q = torch.empty((B, Hq, D), device="cuda", dtype=torch.bfloat16)
+    k = torch.empty((B, L, Hkv, D), device="cuda", dtype=torch.bfloat16)
+    v = torch.empty_like(k)
+    lens = torch.tensor([3000, 1777, 1, 640], device="cuda", dtype=torch.int32)
+    o_g = torch.empty_like(q)
+    lse_g = torch.empty((B, Hq), device="cuda", dtype=torch.float32)
+
+    def fill(seed):
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        for t in (q, k, v):
+            t.copy_(torch.randn(t.shape, generator=g, device="cuda", dtype=torch.float32).to(t.dtype))
+
+    a = _args(q, k, v, o_g, lse_g, lens, 512)
+    fill(1)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    st = C.c_void_p(side.cuda_stream)
+    _lib.check(lib.mi_decode_noalloc(C.byref(a), st))      # first call on this device: outside capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        _lib.check(lib.mi_decode_noalloc(C.byref(a), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    for rep in range(4):
+        fill(10 + rep)
+        if rep == 2:
+            lens.copy_(torch.tensor([5, 2999, 0, 64], device="cuda", dtype=torch.int32))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got_o, got_lse = o_g.clone(), lse_g.clone()
+        o = torch.full_like(q, float("nan"))
+        lse = torch.full_like(lse_g, float("nan"))
+        b = _lib.DecodeArgs.from_buffer_copy(a)
+        b.o, b.lse = o.data_ptr(), lse.data_ptr()
+        nbytes = lib.mi_decode_workspace_bytes(C.byref(b))
+        ws = torch.empty(nbytes, device="cuda", dtype=torch.uint8)
+        b.workspace, b.workspace_bytes = ws.data_ptr(), nbytes
+        _lib.check(lib.mi_decode(C.byref(b), None))
+        torch.cuda.synchronize()
+        assert torch.equal(got_o, o) and torch.equal(got_lse, lse), rep

@@ -9,7 +9,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmi_attn.so")
 
-MI_ATTN_ABI_VERSION = 5
+MI_ATTN_ABI_VERSION = 6
 MI_DECODE_STATIC_SCRATCH_BYTES = 32 << 20
 MI_KV_BATCHED, MI_KV_PACKED, MI_KV_PAGED = 0, 1, 2
 MI_ATTN_BLOCK = 64
@@ -49,7 +49,7 @@ class AttnFwdArgs(C.Structure):
         ("cu_seqlens", _vp),
         ("batch", _i32), ("heads_q", _i32), ("heads_kv", _i32),
         ("max_seqlen", _i32), ("head_dim", _i32), ("causal", _i32),
-        ("scale_log2", _f32),
+        ("scale_log2", _f32), ("total_rows", _i32),
     ]
 
 
@@ -68,7 +68,7 @@ class AttnSparseArgs(C.Structure):
         ("batch", _i32), ("heads_q", _i32), ("heads_kv", _i32),
         ("max_seqlen", _i32), ("head_dim", _i32), ("block_size", _i32),
         ("window_local", _i32), ("window_global", _i32),
-        ("scale_log2", _f32),
+        ("scale_log2", _f32), ("total_rows", _i32),
     ]
 
 
@@ -83,7 +83,7 @@ class AttnBwdArgs(C.Structure):
            ("batch", _i32), ("heads_q", _i32), ("heads_kv", _i32),
            ("max_seqlen", _i32), ("head_dim", _i32), ("causal", _i32),
            ("scale_log2", _f32),
-           ("workspace", _vp), ("workspace_bytes", _sz)]
+           ("workspace", _vp), ("workspace_bytes", _sz), ("total_rows", _i32)]
     )
 
 
@@ -149,6 +149,7 @@ class DecodeArgs(C.Structure):
         ("include_last_block", _i32),
         ("kv_layout", _i32), ("page_size", _i32),
         ("page_table", _vp), ("page_table_stride_b", _i64),
+        ("window_form", _i32),
     ]
 
 

@@ -22,6 +22,17 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+// packed outputs [row][head][head_dim] (+ fp32 lse [row][head]) -> fill descriptors
+mi::RowFillTensor fill_of(void* base, int64_t stride_s, int64_t stride_h, int heads, int elem_bytes, int row_elems) {
+  mi::RowFillTensor t;
+  t.base = base;
+  t.row_stride = stride_s * elem_bytes;
+  t.head_stride = stride_h * elem_bytes;
+  t.heads = heads;
+  t.bytes = row_elems * elem_bytes;
+  return t;
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 bool mult8(int64_t s) { return (s % 8) == 0; }
 
@@ -79,8 +90,10 @@ void fill_prefill(const A* a, mi::PrefillParams& p, int rows_per_wg) {
   p.win_local = -1; p.win_global = -1;
 }
 
+bool decode_listed(const mi_decode_args* a) { return a->block_idx != nullptr || a->window_form == 1; }
+
 int decode_splits(const mi_decode_args* a) {
-  if (a->block_idx) return (a->max_blocks + (a->include_last_block ? 1 : 0) + a->split_blocks - 1) / a->split_blocks;
+  if (decode_listed(a)) return (a->max_blocks + ((a->include_last_block && a->window_form != 1) ? 1 : 0) + a->split_blocks - 1) / a->split_blocks;
   return (a->max_seqlen + a->split_tokens - 1) / a->split_tokens;
 }
 
@@ -98,13 +111,16 @@ void fill_decode(const mi_decode_args* a, mi::DecodeParams& p) {
   p.n_splits = decode_splits(a);
   p.part_o = static_cast<float*>(a->workspace);
   p.part_lse = p.part_o + (size_t)a->batch * a->heads_q * p.n_splits * a->head_dim;
+  p.gslices = (a->heads_q / a->heads_kv + 31) / 32;
+  const bool listed = decode_listed(a);
+  p.list_mode = a->window_form == 1 ? 2 : (a->block_idx ? 1 : 0);
   p.block_idx = a->block_idx; p.block_cnt = a->block_cnt;
   p.bi_sb = a->block_idx_stride_b; p.bi_sh = a->block_idx_stride_h;
   p.max_blocks = a->max_blocks; p.split_blocks = a->split_blocks;
-  p.win_local = a->block_idx ? a->window_local : -1;
-  p.win_global = a->block_idx ? a->window_global : -1;
-  p.add_last = (a->block_idx && a->include_last_block) ? 1 : 0;
-  if (!a->block_idx) { p.max_blocks = 0; p.split_blocks = 1; }
+  p.win_local = listed ? a->window_local : -1;
+  p.win_global = listed ? a->window_global : -1;
+  p.add_last = (p.list_mode == 1 && a->include_last_block) ? 1 : 0;
+  if (!listed) { p.max_blocks = 0; p.split_blocks = 1; }
   p.kv_layout = a->kv_layout; p.page_size = a->page_size;
   p.page_table = a->page_table; p.pt_sb = a->page_table_stride_b;
 }
@@ -114,7 +130,23 @@ int launch_status(int hip_err, const char* what) {
   return fail(MI_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(static_cast<hipError_t>(hip_err)));
 }
 
+// total_rows > 0: zero the rows of o and lse that belong to no sequence
+template <typename A>
+int zero_uncovered(const A* a, hipStream_t s) {
+  if (a->total_rows <= 0) return MI_OK;
+  mi::RowFillParams f;
+  std::memset(&f, 0, sizeof(f));
+  f.cu = a->cu_seqlens; f.batch = a->batch; f.total_rows = a->total_rows; f.max_seqlen = a->max_seqlen;
+  f.t[f.n_tensors++] = fill_of(a->o, a->o_stride_s, a->o_stride_h, a->heads_q, 2, a->head_dim);
+  if (a->lse) f.t[f.n_tensors++] = fill_of(a->lse, a->lse_stride_s, a->lse_stride_h, a->heads_q, 4, 1);
+  return launch_status(mi::launch_zero_uncovered_rows(f, s), "zero fill of rows outside every sequence");
+}
+
 }  // namespace
+
+namespace mi {
+int set_error(int code, const char* msg) { return fail(code, "%s", msg); }
+}  // namespace mi
 
 extern "C" {
 
@@ -150,6 +182,8 @@ int mi_attn_fwd_validate(const mi_attn_fwd_args* a) {
   if ((rc = check_qkvo(a))) return rc;
   if ((rc = check_prefill_strides(a))) return rc;
   if (a->causal != 0 && a->causal != 1) return fail(MI_ERR_SHAPE, "causal must be 0 or 1");
+  if (a->total_rows < 0) return fail(MI_ERR_SHAPE, "total_rows %d is negative", a->total_rows);
+  if (a->total_rows > 0 && !a->cu_seqlens) return fail(MI_ERR_SHAPE, "total_rows is for the packed form (cu_seqlens != NULL)");
   // (work item ids are 32-bit and the persistent kernel steps them by its grid size)
   const long long wgs = (((long long)a->max_seqlen + mi::kDenseRows - 1) / mi::kDenseRows) * a->heads_q * a->batch;
   if (wgs > 0x3fffffffLL) return fail(MI_ERR_SHAPE, "%lld work items are too many", wgs);
@@ -327,7 +361,9 @@ int mi_attn_bwd_validate(const mi_attn_bwd_args* a) {
     return fail(MI_ERR_STRUCT_SIZE, "mi_attn_bwd_args.struct_size %u != %zu", a->struct_size, sizeof(mi_attn_bwd_args));
   int rc = check_common(a->dtype, a->head_dim, a->batch, a->heads_q, a->heads_kv, a->max_seqlen, a->scale_log2);
   if (rc) return rc;
-  if (a->max_seqlen == 0) return MI_OK;
+  if (a->total_rows < 0) return fail(MI_ERR_SHAPE, "total_rows %d is negative", a->total_rows);
+  if (a->total_rows > 0 && !a->cu_seqlens) return fail(MI_ERR_SHAPE, "total_rows is for the packed form (cu_seqlens != NULL)");
+  if (a->max_seqlen == 0 && a->total_rows == 0) return MI_OK;
   const void* ptrs[] = {a->q, a->k, a->v, a->o, a->dout, a->lse, a->dq, a->dk, a->dv};
   for (const void* x : ptrs)
     if (!x) return fail(MI_ERR_NULL_POINTER, "q, k, v, o, dout, lse, dq, dk and dv must be non-NULL");
@@ -354,9 +390,11 @@ int mi_attn_bwd_validate(const mi_attn_bwd_args* a) {
   const long long wgs = (long long)((a->max_seqlen + 255) / 256) * a->heads_q * a->batch;
   if (wgs > 0x7fffffffLL || a->heads_q > 65535 || a->batch > 65535)
     return fail(MI_ERR_SHAPE, "launch grid too large");
-  if (!a->workspace || a->workspace_bytes < mi_attn_bwd_workspace_bytes(a))
-    return fail(MI_ERR_WORKSPACE, "workspace of %zu bytes needed", mi_attn_bwd_workspace_bytes(a));
-  if (!aligned16(a->workspace)) return fail(MI_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
+  if (a->max_seqlen > 0) {
+    if (!a->workspace || a->workspace_bytes < mi_attn_bwd_workspace_bytes(a))
+      return fail(MI_ERR_WORKSPACE, "workspace of %zu bytes needed", mi_attn_bwd_workspace_bytes(a));
+    if (!aligned16(a->workspace)) return fail(MI_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
+  }
   return MI_OK;
 }
 
@@ -368,6 +406,17 @@ size_t mi_attn_bwd_workspace_bytes(const mi_attn_bwd_args* a) {
 int mi_attn_bwd(const mi_attn_bwd_args* a, void* stream) {
   int rc = mi_attn_bwd_validate(a);
   if (rc) return rc;
+  if (a->total_rows > 0) {
+    mi::RowFillParams f;
+    std::memset(&f, 0, sizeof(f));
+    f.cu = a->cu_seqlens; f.batch = a->batch; f.total_rows = a->total_rows; f.max_seqlen = a->max_seqlen;
+    f.t[f.n_tensors++] = fill_of(a->dq, a->dq_stride_s, a->dq_stride_h, a->heads_q, 2, a->head_dim);
+    f.t[f.n_tensors++] = fill_of(a->dk, a->dk_stride_s, a->dk_stride_h, a->heads_kv, 2, a->head_dim);
+    f.t[f.n_tensors++] = fill_of(a->dv, a->dv_stride_s, a->dv_stride_h, a->heads_kv, 2, a->head_dim);
+    if ((rc = launch_status(mi::launch_zero_uncovered_rows(f, static_cast<hipStream_t>(stream)),
+                            "zero fill of rows outside every sequence")))
+      return rc;
+  }
   if (a->max_seqlen == 0) return MI_OK;
   mi::BwdParams p;
   std::memset(&p, 0, sizeof(p));
@@ -396,6 +445,7 @@ int mi_attn_bwd(const mi_attn_bwd_args* a, void* stream) {
 int mi_attn_fwd(const mi_attn_fwd_args* a, void* stream) {
   int rc = mi_attn_fwd_validate(a);
   if (rc) return rc;
+  if ((rc = zero_uncovered(a, static_cast<hipStream_t>(stream)))) return rc;
   if (a->max_seqlen == 0) return MI_OK;
   mi::PrefillParams p;
   fill_prefill(a, p, mi::kDenseRows);
@@ -417,6 +467,8 @@ int mi_attn_fwd_blocksparse_validate(const mi_attn_sparse_args* a) {
     return fail(MI_ERR_SPARSE_LAYOUT, "mask strides must be >= 0");
   if ((a->window_local < 0) != (a->window_global < 0) || a->window_local < -1 || a->window_global < -1)
     return fail(MI_ERR_SPARSE_LAYOUT, "window_local/window_global must both be -1 or both be >= 0");
+  if (a->total_rows < 0) return fail(MI_ERR_SHAPE, "total_rows %d is negative", a->total_rows);
+  if (a->total_rows > 0 && !a->cu_seqlens) return fail(MI_ERR_SHAPE, "total_rows is for the packed form (cu_seqlens != NULL)");
   const long long wgs = (((long long)a->max_seqlen + mi::kSparseRows - 1) / mi::kSparseRows) * a->heads_q * a->batch;
   if (wgs > 0x7fffffffLL) return fail(MI_ERR_SHAPE, "grid of %lld workgroups is too large", wgs);
   return MI_OK;
@@ -425,6 +477,7 @@ int mi_attn_fwd_blocksparse_validate(const mi_attn_sparse_args* a) {
 int mi_attn_fwd_blocksparse(const mi_attn_sparse_args* a, void* stream) {
   int rc = mi_attn_fwd_blocksparse_validate(a);
   if (rc) return rc;
+  if ((rc = zero_uncovered(a, static_cast<hipStream_t>(stream)))) return rc;
   if (a->max_seqlen == 0) return MI_OK;
   mi::PrefillParams p;
   fill_prefill(a, p, mi::kSparseRows);
@@ -444,9 +497,16 @@ static int decode_validate_shape(const mi_decode_args* a) {
     return fail(MI_ERR_STRUCT_SIZE, "mi_decode_args.struct_size %u != %zu", a->struct_size, sizeof(mi_decode_args));
   int rc = check_common(a->dtype, a->head_dim, a->batch, a->heads_q, a->heads_kv, a->max_seqlen, a->scale_log2);
   if (rc) return rc;
-  if (a->heads_q / a->heads_kv > 32)
-    return fail(MI_ERR_GQA, "at most 32 query heads per kv head (got %d)", a->heads_q / a->heads_kv);
-  if (a->block_idx) {
+  if (a->window_form != 0 && a->window_form != 1) return fail(MI_ERR_SPARSE_LAYOUT, "window_form must be 0 or 1");
+  if (a->window_form == 1) {
+    if (a->block_size != MI_ATTN_BLOCK) return fail(MI_ERR_SPARSE_LAYOUT, "block_size %d must be %d", a->block_size, MI_ATTN_BLOCK);
+    if (a->window_local < 0 || a->window_global < 0)
+      return fail(MI_ERR_SPARSE_LAYOUT, "the window form needs window_local and window_global >= 0");
+    const long long need = ((long long)a->window_global + 63) / 64 + ((long long)a->window_local + 63) / 64 + 1;
+    if (a->max_blocks < need || a->split_blocks <= 0)
+      return fail(MI_ERR_SPARSE_LAYOUT, "the window form needs max_blocks >= %lld (got %d) and split_blocks > 0 (got %d)",
+                  need, a->max_blocks, a->split_blocks);
+  } else if (a->block_idx) {
     if (a->block_size != MI_ATTN_BLOCK) return fail(MI_ERR_SPARSE_LAYOUT, "block_size %d must be %d", a->block_size, MI_ATTN_BLOCK);
     if (a->include_last_block != 0 && a->include_last_block != 1)
       return fail(MI_ERR_SPARSE_LAYOUT, "include_last_block must be 0 or 1");
@@ -468,7 +528,7 @@ static int decode_validate_shape(const mi_decode_args* a) {
     return fail(MI_ERR_SHAPE, "paged KV needs page_size a positive multiple of 32 (got %d) and a page table stride >= 0",
                 a->page_size);
   if (decode_splits(a) > 65535) return fail(MI_ERR_WORKSPACE, "more than 65535 splits per sequence");
-  if (a->heads_kv > 65535 || a->batch > 65535 || a->heads_q > 0x7fffffff / 2)
+  if ((long long)a->heads_kv * ((a->heads_q / a->heads_kv + 31) / 32) > 65535 || a->batch > 65535 || a->heads_q > 0x7fffffff / 2)
     return fail(MI_ERR_SHAPE, "batch / head count exceeds the launch grid limits");
   return MI_OK;
 }

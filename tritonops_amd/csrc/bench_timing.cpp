@@ -3,11 +3,13 @@
 #include <hip/hip_runtime.h>
 
 #include "../../include/mi_attn_bench.h"
+#include "kernels.h"
 
 extern "C" int mi_time_launches(int kind, const void* args, int n_args, size_t arg_stride, void* stream, int warmup,
                                 int iters, float* ms_per_launch) {
-  if (!args || !ms_per_launch || n_args <= 0 || iters <= 0 || warmup < 0 || kind < 0 || kind > 11)
-    return MI_ERR_SHAPE;
+  if (!args || !ms_per_launch) return mi::set_error(MI_ERR_NULL_POINTER, "mi_time_launches: args and ms_per_launch must be non-NULL");
+  if (n_args <= 0 || iters <= 0 || warmup < 0 || kind < 0 || kind > 11)
+    return mi::set_error(MI_ERR_SHAPE, "mi_time_launches: n_args and iters must be positive, warmup >= 0, kind in [0, 11]");
   const char* base = static_cast<const char*>(args);
   int n = 0;
   auto once = [&]() -> int {
@@ -33,10 +35,10 @@ extern "C" int mi_time_launches(int kind, const void* args, int n_args, size_t a
     if (rc) return rc;
   }
   hipEvent_t e0, e1;
-  if (hipEventCreate(&e0) != hipSuccess) return MI_ERR_NO_DEVICE;
+  if (hipEventCreate(&e0) != hipSuccess) return mi::set_error(MI_ERR_NO_DEVICE, "mi_time_launches: hipEventCreate failed");
   if (hipEventCreate(&e1) != hipSuccess) {
     (void)hipEventDestroy(e0);
-    return MI_ERR_NO_DEVICE;
+    return mi::set_error(MI_ERR_NO_DEVICE, "mi_time_launches: hipEventCreate failed");
   }
   int rc = MI_OK;
   (void)hipEventRecord(e0, s);
@@ -47,8 +49,8 @@ extern "C" int mi_time_launches(int kind, const void* args, int n_args, size_t a
   if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
   (void)hipEventDestroy(e0);
   (void)hipEventDestroy(e1);
-  if (rc) return rc;
-  if (e != hipSuccess) return MI_ERR_LAUNCH;
+  if (rc) return rc;  // the entry point that failed has set the message
+  if (e != hipSuccess) return mi::set_error(MI_ERR_LAUNCH, hipGetErrorString(e));
   *ms_per_launch = ms / iters;
   return MI_OK;
 }

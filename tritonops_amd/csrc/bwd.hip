@@ -157,7 +157,8 @@ __device__ __forceinline__ void bwd_dq_item(const BwdParams& p, const int bid) {
   int64_t start;  // first row of the sequence in packed tensors
   if (p.cu) {
     start = p.cu[b];
-    len = p.cu[b + 1] - (int)start;
+    // never beyond the bound the workspace and the grid were sized for
+    len = min(p.cu[b + 1] - (int)start, p.max_seqlen);
   } else {
     start = 0;
     len = p.max_seqlen;
@@ -544,7 +545,8 @@ __device__ __forceinline__ void bwd_dkdv_item(const BwdParams& p, const int bid,
   int64_t start;
   if (p.cu) {
     start = p.cu[b];
-    len = p.cu[b + 1] - (int)start;
+    // never beyond the bound the workspace and the grid were sized for
+    len = min(p.cu[b + 1] - (int)start, p.max_seqlen);
   } else {
     start = 0;
     len = p.max_seqlen;
@@ -1114,8 +1116,8 @@ int launch_dq(const BwdParams& p, hipStream_t s) {
   constexpr size_t lds = kBwdStages * (2 * 64 * 256 + 1024);
   static_assert(lds >= 8 * 32 * (D * 2 + 16), "epilogue staging must fit the tile ring");
   auto kern = bwd_dq_kernel<T, D>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  if (e != hipSuccess) return (int)e;
+  static LdsLimitOnce lds_once;
+  if (const int e = raise_lds_limit(lds_once, reinterpret_cast<const void*>(kern), (int)lds)) return e;
   const long long items = (long long)p.n_rtiles * p.hq * p.batch;
   long long grid = items;
   const int cus = device_cu_count();
@@ -1129,8 +1131,8 @@ int launch_dkdv(const BwdParams& p, hipStream_t s) {
   constexpr size_t lds = kBwdStages * (2 * 64 * 256 + 1024) + 2 * 4 * 2 * 2048;  // tile ring + P exchange
   static_assert(lds >= 8 * 32 * (D * 2 + 16), "epilogue staging must fit");
   auto kern = bwd_dkdv_kernel<T, D>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  if (e != hipSuccess) return (int)e;
+  static LdsLimitOnce lds_once;
+  if (const int e = raise_lds_limit(lds_once, reinterpret_cast<const void*>(kern), (int)lds)) return e;
   const int n_rt = (p.max_seqlen + 127) / 128;
   const long long items = (long long)n_rt * p.hkv * p.batch;
   long long grid = items;

@@ -14,7 +14,8 @@
 // prefill kernel uses, so each K/V byte is fetched once for the whole group
 // (the reference launches one program per q-head and re-reads KV G times,
 // flash_attn_decoding.py:42-45,264-268) and the dot products cost no VALU
-// work.  KV streams global -> registers -> wave-private LDS in 32-key tiles
+// work.  A group of more than 32 heads is split into slices of 32, each a work
+// item of its own: KV is then fetched once per slice.  KV streams global -> registers -> wave-private LDS in 32-key tiles
 // with fully coalesced 16-byte loads (non-temporal: every byte is used once);
 // as soon as a tile has arrived, each register is written to LDS and refilled
 // with its part of the tile after next.  No barriers are needed because a
@@ -37,10 +38,31 @@ namespace {
 
 constexpr int kDecTile = 32;
 
-// One work item: chunk `split` of (sequence b, kv-head kvh).
+// The block list of the window form, which is arithmetic: the blocks of the
+// first `wg` tokens (entries 0 .. n_sink-1), then the blocks from token
+// max(len - wl, 0) to the last one (entries n_sink .. cnt-1, starting at block
+// tail0), every block once.
+struct WindowList {
+  int n_sink, tail0, cnt;
+  __device__ __forceinline__ int block(int e) const { return e < n_sink ? e : tail0 + (e - n_sink); }
+};
+__device__ __forceinline__ WindowList window_list(int len, int wg, int wl) {
+  const int nblk = (len + 63) / 64;
+  WindowList w;
+  w.n_sink = min((wg + 63) / 64, nblk);
+  w.tail0 = max(max(len - wl, 0) / 64, w.n_sink);
+  w.cnt = w.n_sink + max(nblk - w.tail0, 0);
+  return w;
+}
+
+// One work item: chunk `split` of (sequence b, kv-head kvh) for the 32 query
+// heads of the group that start at head g0 of it (slice kvs % gslices; a group
+// of up to 32 heads is one slice).
 template <typename T, int D>
-__device__ __forceinline__ void decode_item(const DecodeParams& p, unsigned char* smem, const int split, const int kvh,
+__device__ __forceinline__ void decode_item(const DecodeParams& p, unsigned char* smem, const int split, const int kvs,
                                             const int b) {
+  const int kvh = kvs / p.gslices;
+  const int g0 = (kvs % p.gslices) * 32;
   using G = RowGeom<D>;
   using F = PaddedFrags<D>;
   constexpr int KTILEB = kDecTile * F::KROWB;
@@ -52,19 +74,29 @@ __device__ __forceinline__ void decode_item(const DecodeParams& p, unsigned char
 
   const int lane = threadIdx.x;
   const int len = p.seq_lens ? p.seq_lens[b] : p.cu[b + 1] - p.cu[b];
-  const int gqa = p.hq / p.hkv;
-  const bool sparse = p.block_idx != nullptr;
+  const int gqa_all = p.hq / p.hkv;
+  const int gqa = min(32, gqa_all - g0);  // query heads of this slice
+  const bool sparse = p.list_mode != 0;
+  const bool derived = p.list_mode == 2;
 
   int n_tiles, t_begin = 0;
   const int32_t* blist = nullptr;
+  WindowList wlist = {0, 0, 0};
   int n_listed = 0;  // listed entries that fall into this chunk
+  int b0 = 0;        // first entry of this chunk
   const int last_blk = (len - 1) / 64;
   if (sparse) {
-    const int cnt = p.block_cnt ? min(p.block_cnt[b * p.hkv + kvh], p.max_blocks) : p.max_blocks;
+    int cnt;
+    if (derived) {
+      wlist = window_list(len, p.win_global, p.win_local);
+      cnt = min(wlist.cnt, p.max_blocks);
+    } else {
+      cnt = p.block_cnt ? min(p.block_cnt[b * p.hkv + kvh], p.max_blocks) : p.max_blocks;
+    }
     const int total = cnt + p.add_last;  // the implicit last block sits behind the list
-    const int b0 = split * p.split_blocks;
+    b0 = split * p.split_blocks;
     if (b0 >= total || len <= 0) return;
-    blist = p.block_idx + b * p.bi_sb + kvh * p.bi_sh + b0;
+    if (!derived) blist = p.block_idx + b * p.bi_sb + kvh * p.bi_sh + b0;
     n_tiles = 2 * min(total - b0, p.split_blocks);
     n_listed = max(0, min(cnt - b0, p.split_blocks));
   } else {
@@ -78,7 +110,7 @@ __device__ __forceinline__ void decode_item(const DecodeParams& p, unsigned char
   auto tile_base = [&](int i) -> int {
     if (!sparse) return t_begin + i * kDecTile;
     const int e = i >> 1;
-    const int blk = e < n_listed ? blist[e] : last_blk;
+    const int blk = e < n_listed ? (derived ? wlist.block(b0 + e) : blist[e]) : last_blk;
     if (p.add_last && e < n_listed && blk == last_blk) return -1;
     return blk * 64 + (i & 1) * kDecTile;
   };
@@ -108,7 +140,7 @@ __device__ __forceinline__ void decode_item(const DecodeParams& p, unsigned char
   i32x4 Qf[G::KSTEPS];
   {
     const T* qr = reinterpret_cast<const T*>(p.q) + b * p.q_sb +
-                  (int64_t)(kvh * gqa + min(lc.lq, gqa - 1)) * p.q_sh + 8 * lc.lh;
+                  (int64_t)(kvh * gqa_all + g0 + min(lc.lq, gqa - 1)) * p.q_sh + 8 * lc.lh;
 #pragma unroll
     for (int c = 0; c < G::KSTEPS; ++c) {
       i32x4 t = *reinterpret_cast<const i32x4*>(qr + 16 * c);
@@ -247,7 +279,7 @@ __device__ __forceinline__ void decode_item(const DecodeParams& p, unsigned char
   const float l_tot = sum_with_other_half(l);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   if (lc.lq < gqa) {
-    const int h = kvh * gqa + lc.lq;
+    const int h = kvh * gqa_all + g0 + lc.lq;
     const int64_t slot = ((int64_t)b * p.hq + h) * p.n_splits + split;
     if (lc.lh == 0) p.part_lse[slot] = l_tot > 0.f ? m + fast_log2(l_tot) : -INFINITY;
     float* po = p.part_o + slot * D;
@@ -273,7 +305,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2)))
 decode_splitkv_kernel(const DecodeParams p) {
   using F = PaddedFrags<D>;
   __shared__ __attribute__((aligned(16))) unsigned char smem[kDecTile * (F::KROWB + F::VROWB)];
-  if (p.block_idx != nullptr) {
+  if (p.list_mode != 0) {
     decode_item<T, D>(p, smem, blockIdx.x, blockIdx.y, blockIdx.z);
     return;
   }
@@ -292,9 +324,10 @@ decode_splitkv_kernel(const DecodeParams p) {
     total += c;
   }
   total = __builtin_amdgcn_readfirstlane(total);
-  const long long items = (long long)total * p.hkv;
+  const int kv_slices = p.hkv * p.gslices;  // (kv-head, 32-head slice of its group) pairs
+  const long long items = (long long)total * kv_slices;
   for (long long g = blockIdx.x; g < items; g += gridDim.x) {
-    const int t = (int)(g / p.hkv), kvh = (int)(g % p.hkv);
+    const int t = (int)(g / kv_slices), kvh = (int)(g % kv_slices);
     // sequence that owns live chunk t: inclusive scan over the chunk counts
     int b = 0, first = 0;
     for (int b0 = 0, seen = 0; b0 < p.batch; b0 += 64) {
@@ -328,9 +361,13 @@ decode_merge_kernel(const DecodeParams p, int D) {
   const int d = threadIdx.x;
   const int len = p.seq_lens ? p.seq_lens[b] : p.cu[b + 1] - p.cu[b];
   int nvalid;
-  if (p.block_idx) {
+  if (p.list_mode != 0) {
     const int kvh = h / (p.hq / p.hkv);
-    const int cnt = p.block_cnt ? min(p.block_cnt[b * p.hkv + kvh], p.max_blocks) : p.max_blocks;
+    int cnt;
+    if (p.list_mode == 2)
+      cnt = min(window_list(len, p.win_global, p.win_local).cnt, p.max_blocks);
+    else
+      cnt = p.block_cnt ? min(p.block_cnt[b * p.hkv + kvh], p.max_blocks) : p.max_blocks;
     nvalid = len > 0 ? (cnt + p.add_last + p.split_blocks - 1) / p.split_blocks : 0;
   } else {
     nvalid = (len + p.split_tokens - 1) / p.split_tokens;
@@ -359,10 +396,10 @@ decode_merge_kernel(const DecodeParams p, int D) {
 
 template <typename T, int D>
 int launch_split(const DecodeParams& p, hipStream_t s) {
-  dim3 grid(p.n_splits, p.hkv, p.batch);
-  if (p.block_idx == nullptr) {
+  dim3 grid(p.n_splits, p.hkv * p.gslices, p.batch);
+  if (p.list_mode == 0) {
     // dense: one resident round (8 wavefronts per CU), fewer when there are fewer chunks
-    const long long slots = (long long)p.n_splits * p.hkv * p.batch;
+    const long long slots = (long long)p.n_splits * p.hkv * p.gslices * p.batch;
     const int cus = device_cu_count();
     const long long resident = 8LL * (cus > 0 ? cus : 256);
     grid = dim3((unsigned)(slots < resident ? slots : resident), 1, 1);

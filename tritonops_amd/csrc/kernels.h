@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace mi {
 
 struct PrefillParams {
@@ -44,8 +46,10 @@ struct DecodeParams {
   int32_t n_splits;      // chunks per sequence (grid.x)
   float* part_o;         // [batch][hq][n_splits][D]
   float* part_lse;       // [batch][hq][n_splits]
+  int32_t gslices;       // slices of 32 query heads per GQA group = ceil((hq / hkv) / 32)
   // block-sparse
-  const int32_t* block_idx;  // null => dense
+  int32_t list_mode;         // 0 dense, 1 block list read from block_idx, 2 list derived from the two windows
+  const int32_t* block_idx;  // list_mode 1
   const int32_t* block_cnt;
   int64_t bi_sb, bi_sh;
   int32_t max_blocks, split_blocks;
@@ -122,6 +126,46 @@ struct XentGradParams {
 
 // CUs of the current device (cached per device; 0 if the query fails).
 int device_cu_count();
+
+// Stores `msg` as this thread's mi_last_error() text and returns `code`
+// (for the host translation units other than api.cpp).
+int set_error(int code, const char* msg);
+
+// Raises a kernel's dynamic-LDS limit to `bytes`, once per (kernel, device):
+// `st` is a state object that belongs to one kernel (a function-local static of
+// its launcher).  Every launch after the first on a device costs one
+// hipGetDevice and records nothing but the kernel launch itself.  Returns
+// hipError_t as int.
+constexpr int kMaxDevices = 64;
+struct LdsLimitOnce {
+  std::atomic<unsigned char> done[kMaxDevices];
+};
+inline int raise_lds_limit(LdsLimitOnce& st, const void* kern, int bytes) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  const bool slot = dev >= 0 && dev < kMaxDevices;
+  if (slot && st.done[dev].load(std::memory_order_acquire)) return 0;
+  e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return (int)e;
+  if (slot) st.done[dev].store(1, std::memory_order_release);
+  return 0;
+}
+
+// Zero-fill of the rows of packed outputs that belong to no sequence: rows of
+// [0, total_rows) behind cu[batch], and rows behind the first max_seqlen tokens
+// of their sequence.  Up to three tensors [row][head][bytes] per call.
+struct RowFillTensor {
+  void* base;
+  int64_t row_stride, head_stride;  // bytes
+  int32_t heads, bytes;             // bytes per (row, head): a multiple of 4
+};
+struct RowFillParams {
+  const int32_t* cu;
+  int32_t batch, total_rows, max_seqlen, n_tensors;
+  RowFillTensor t[3];
+};
+int launch_zero_uncovered_rows(const RowFillParams& p, hipStream_t s);
 
 // dtype: 0 bf16, 1 f16.  head_dim in {64, 96, 128}.  Return hipError_t as int.
 int launch_prefill_dense(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);

@@ -66,7 +66,8 @@ __device__ __forceinline__ bool item_geo(const PrefillParams& p, const int bid, 
   g.h = g.kvh * gqa + s % gqa;
   if (p.cu) {
     const int start = p.cu[g.b];
-    g.len = p.cu[g.b + 1] - start;
+    // (a sequence longer than the caller's bound is cut at the bound: the grid covers no row beyond it)
+    g.len = min(p.cu[g.b + 1] - start, p.max_seqlen);
     g.q_off = start * p.q_ss;
     g.k_off = start * p.k_ss;
     g.v_off = start * p.v_ss;
@@ -1090,9 +1091,8 @@ int launch_one(const PrefillParams& p, hipStream_t s) {
   else
     kern = dense_kernel<T, D>;
   constexpr size_t lds = prefill_lds_bytes<D, NW, NS, TN>();
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  if (e != hipSuccess) return (int)e;
+  static LdsLimitOnce lds_once;
+  if (const int e = raise_lds_limit(lds_once, reinterpret_cast<const void*>(kern), (int)lds)) return e;
   PrefillParams pp = p;
   const long long items = (long long)p.n_qtiles * p.hq * p.batch;
   pp.n_items = (int)items;
@@ -1127,7 +1127,46 @@ int dispatch(const PrefillParams& p, int dtype, int head_dim, hipStream_t s) {
   return (int)hipErrorInvalidValue;
 }
 
+// Rows of packed outputs that no work item writes.  A workgroup looks at 64
+// consecutive rows: lane i finds the sequence of row r0 + i by bisection of cu
+// (non-decreasing) and the workgroup leaves at once when all 64 are covered,
+// which is the usual case; otherwise its threads zero the uncovered rows.
+__global__ void __launch_bounds__(256) zero_uncovered_rows_kernel(const RowFillParams p) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 64 + lane;
+  bool uncovered = false;
+  if (row < p.total_rows) {
+    // last b in [0, batch] with cu[b] <= row
+    int lo = 0, hi = p.batch;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (p.cu[mid] <= row) lo = mid; else hi = mid - 1;
+    }
+    uncovered = lo >= p.batch || row < p.cu[0] || row - p.cu[lo] >= p.max_seqlen;
+  }
+  const unsigned long long todo = __builtin_amdgcn_ballot_w64(uncovered);
+  if (todo == 0) return;
+  for (int i = 0; i < 64; ++i) {
+    if (!((todo >> i) & 1)) continue;
+    const int64_t r = (int64_t)blockIdx.x * 64 + i;
+    for (int k = 0; k < p.n_tensors; ++k) {
+      const RowFillTensor& t = p.t[k];
+      const int words = t.bytes >> 2;
+      for (int j = threadIdx.x; j < t.heads * words; j += blockDim.x) {
+        const int h = j / words, w = j % words;
+        *reinterpret_cast<uint32_t*>(static_cast<char*>(t.base) + r * t.row_stride + h * t.head_stride + 4 * w) = 0u;
+      }
+    }
+  }
+}
+
 }  // namespace
+
+int launch_zero_uncovered_rows(const RowFillParams& p, hipStream_t s) {
+  if (p.total_rows <= 0 || p.n_tensors <= 0) return 0;
+  hipLaunchKernelGGL(zero_uncovered_rows_kernel, dim3((unsigned)((p.total_rows + 63) / 64)), dim3(256), 0, s, p);
+  return (int)hipGetLastError();
+}
 
 // CUs of the current device (cached per device; 0 if the query fails)
 int device_cu_count() {

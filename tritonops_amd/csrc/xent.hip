@@ -461,8 +461,8 @@ namespace {
 template <typename T, bool GRAD>
 int launch_gemm(const XentParams& p, unsigned grid, hipStream_t s) {
   auto kern = xent_gemm_kernel<T, GRAD>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kXLdsBytes);
-  if (e != hipSuccess) return (int)e;
+  static LdsLimitOnce lds_once;
+  if (const int e = raise_lds_limit(lds_once, reinterpret_cast<const void*>(kern), kXLdsBytes)) return e;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(512), kXLdsBytes, s, p);
   return (int)hipGetLastError();
 }

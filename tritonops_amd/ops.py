@@ -7,6 +7,7 @@ is no fallback: without the built library every call raises.
 """
 import ctypes as C
 import math
+import weakref
 
 import torch
 
@@ -53,12 +54,30 @@ def _ptr(t):
     return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
 
 
+_MAX_LEN_CACHE = {}   # id(cu tensor) -> (weak reference, version counter, longest sequence)
+
+
 def _max_len(cu_seq_lens, max_seq_len):
+    """Longest sequence of the batch, which sizes the launch.  Without a hint
+    it costs the host round trip the reference launcher makes on every call
+    (flash_attn_triton/flash_attn_triton.py:621); here the answer is kept per
+    cu_seq_lens tensor OBJECT for as long as that object lives and its version
+    counter (bumped by every in-place write) has not moved, so the layers of a
+    model that share one cu_seq_lens pay for it once per batch."""
     if max_seq_len is not None:
         return int(max_seq_len)
-    # same host round trip as the reference launcher
-    # (flash_attn_triton/flash_attn_triton.py:621)
-    return int((cu_seq_lens[1:] - cu_seq_lens[:-1]).max().item())
+    key = id(cu_seq_lens)
+    hit = _MAX_LEN_CACHE.get(key)
+    if hit is not None and hit[0]() is cu_seq_lens and hit[1] == cu_seq_lens._version:
+        return hit[2]
+    n = int((cu_seq_lens[1:] - cu_seq_lens[:-1]).max().item())
+    if len(_MAX_LEN_CACHE) >= 256:
+        _MAX_LEN_CACHE.clear()
+    try:
+        _MAX_LEN_CACHE[key] = (weakref.ref(cu_seq_lens), cu_seq_lens._version, n)
+    except TypeError:
+        pass
+    return n
 
 
 _HEAD_DIMS = (64, 96, 128)
@@ -72,7 +91,11 @@ def _padded_head_dim(D):
     for d in _HEAD_DIMS:
         if D <= d:
             return d
-    raise ValueError("head_dim %d is not supported (at most %d)" % (D, _HEAD_DIMS[-1]))
+    raise ValueError(
+        "head_dim %d exceeds %d, the widest row the gfx950 kernels of this library are built for (rows of 64, 96 "
+        "and 128 elements; smaller head_dims are zero-padded to the next of them).  The reference pads any "
+        "head_dim to a power of two and tiles the value dimension by 128 (flash_attn_triton.py:612,622); nothing "
+        "wider is implemented here, and no device work has been started." % (D, _HEAD_DIMS[-1]))
 
 
 def _pad_last(t, Dp):
@@ -129,13 +152,11 @@ def _dense_fwd(q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, want_lse=T
     if bhsd:
         o = torch.empty((X, Hq, S, D), device=q.device, dtype=q.dtype).transpose(1, 2)
         lse = torch.empty((X, Hq, S), device=q.device, dtype=torch.float32).transpose(1, 2) if want_lse else None
-    elif packed:
-        # rows outside every sequence (padding behind cu_seq_lens[-1]) are never
-        # written by the kernel: the reference zero-fills both outputs
-        # (flash_attn_triton.py:608-609)
-        o = torch.zeros((X, S, Hq, D), device=q.device, dtype=q.dtype)
-        lse = torch.zeros((X, S, Hq), device=q.device, dtype=torch.float32) if want_lse else None
     else:
+        # packed: rows outside every sequence (padding behind cu_seq_lens[-1]) are
+        # zero in the reference, which zero-fills both outputs first
+        # (flash_attn_triton.py:608-609); here the library zeroes just those rows
+        # (total_rows below)
         o = torch.empty((X, S, Hq, D), device=q.device, dtype=q.dtype)
         lse = torch.empty((X, S, Hq), device=q.device, dtype=torch.float32) if want_lse else None
     if q.numel() == 0:
@@ -150,7 +171,8 @@ def _dense_fwd(q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, want_lse=T
         cu = cu_seq_lens.to(torch.int32)
         a.cu_seqlens = _ptr(cu)
         a.batch = cu.numel() - 1
-        a.max_seqlen = min(_max_len(cu, max_seq_len), S)
+        a.max_seqlen = min(_max_len(cu_seq_lens, max_seq_len), S)
+        a.total_rows = S
     else:
         a.cu_seqlens = None
         a.batch = X
@@ -199,9 +221,8 @@ def _dense_bwd(q, k, v, o, do, lse, cu_seq_lens, scale_log2, causal, max_seq_len
         cu = cu_seq_lens.to(torch.int32)
         a.cu_seqlens = _ptr(cu)
         a.batch = cu.numel() - 1
-        a.max_seqlen = min(_max_len(cu, max_seq_len), S)
-        # rows outside every sequence receive no gradient
-        dq.zero_(), dk.zero_(), dv.zero_()
+        a.max_seqlen = min(_max_len(cu_seq_lens, max_seq_len), S)
+        a.total_rows = S  # rows outside every sequence receive zeros
     else:
         a.cu_seqlens = None
         a.batch = X
@@ -234,8 +255,8 @@ def flash_attn_triton_fwd(q, k, v, cu_seq_lens, sm_scale, *, max_seq_len=None):
     (:839).  Returns (o [1,T,Hq,D], lse [1,T,Hq] fp32, base 2).  Rows outside
     every sequence are zero in both, as in the reference (:608-609).
     `max_seq_len` skips the host sync that sizes the grid (:621); it must be
-    an upper bound of every sequence length (rows beyond it may or may not be
-    computed).
+    an upper bound of every sequence length: a longer sequence is cut at the
+    bound (its later rows are not attended and come back as zeros).
     """
     return _dense_fwd(q, k, v, cu_seq_lens, sm_scale, True, max_seq_len)
 
@@ -248,7 +269,8 @@ class flash_attn_triton(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, cu_seq_lens):
         sm_scale = (1 / q.shape[-1]) ** 0.5 * LOG2E
-        o, lse = flash_attn_triton_fwd(q, k, v, cu_seq_lens, sm_scale)
+        ctx.max_len = _max_len(cu_seq_lens, None)   # once: the backward gets the saved tensors as new objects
+        o, lse = flash_attn_triton_fwd(q, k, v, cu_seq_lens, sm_scale, max_seq_len=ctx.max_len)
         ctx.save_for_backward(q, k, v, o, lse, cu_seq_lens)
         ctx.sm_scale = sm_scale
         return o
@@ -256,7 +278,7 @@ class flash_attn_triton(torch.autograd.Function):
     @staticmethod
     def backward(ctx, do):
         q, k, v, o, lse, cu_seq_lens = ctx.saved_tensors
-        dq, dk, dv = flash_attn_triton_bwd(q, k, v, o, do, lse, cu_seq_lens, ctx.sm_scale)
+        dq, dk, dv = flash_attn_triton_bwd(q, k, v, o, do, lse, cu_seq_lens, ctx.sm_scale, max_seq_len=ctx.max_len)
         return dq, dk, dv, None
 
 
@@ -267,6 +289,8 @@ class _FlashAttention(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, bhsd):
+        if cu_seq_lens is not None and max_seq_len is None:
+            max_seq_len = _max_len(cu_seq_lens, None)
         o, lse = _dense_fwd(q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, True, bhsd)
         ctx.save_for_backward(q, k, v, o, lse, cu_seq_lens)
         ctx.opts = (scale_log2, causal, max_seq_len)
@@ -357,11 +381,12 @@ def flash_attn_sparse_triton(q, k, v, cu_seqlens, softmax_scale=None, local_wind
         if X != 1:
             raise ValueError("packed layout expects a leading dimension of 1")
         cu = cu_seqlens.to(torch.int32)
-        max_len = min(_max_len(cu, max_seq_len), T)
-        # rows outside every sequence are not written by the kernel; zero like the
-        # reference (flash_attn_sparse_attn_triton.py:274-275)
-        o = torch.zeros_like(q)
-        lse = torch.zeros((1, T, Hq), device=q.device, dtype=torch.float32)
+        max_len = min(_max_len(cu_seqlens, max_seq_len), T)
+        # rows outside every sequence are zero in the reference, which zero-fills
+        # both outputs (flash_attn_sparse_attn_triton.py:274-275); the library
+        # zeroes just those rows (total_rows below)
+        o = torch.empty_like(q)
+        lse = torch.empty((1, T, Hq), device=q.device, dtype=torch.float32)
         qv, kv, vv, ov, lv = q, k, v, o, lse
         batch = cu.numel() - 1
     else:
@@ -401,13 +426,15 @@ def flash_attn_sparse_triton(q, k, v, cu_seqlens, softmax_scale=None, local_wind
     a.block_size = _masks.BLOCK
     a.window_local, a.window_global = wl, wg
     a.scale_log2 = scale
+    a.total_rows = T if packed else 0
     _lib.check(lib.mi_attn_fwd_blocksparse(C.byref(a), _stream()))
     return o, lse
 
 
 def _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, return_lse,
             block_idx=None, block_cnt=None, bi_strides=(0, 0), max_blocks=0, split_blocks=0,
-            window=(-1, -1), include_last=False, kv_layout="batched", page_table=None, page_size=0):
+            window=(-1, -1), include_last=False, kv_layout="batched", page_table=None, page_size=0,
+            window_form=False):
     if q.dim() != 3 or k.dim() != 4:
         raise ValueError("decoding takes q [B, Hq, D] and k, v [B, maxL, Hkv, D] (or a packed / paged cache)")
     if v.shape != k.shape:
@@ -432,7 +459,7 @@ def _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, re
         Dp = _padded_head_dim(D0)
         out = _decode(_pad_last(q, Dp), _pad_last(k, Dp), _pad_last(v, Dp), cu_seq_lens, seq_lens, scale, max_seq_len,
                       split_tokens, return_lse, block_idx, block_cnt, bi_strides, max_blocks, split_blocks, window,
-                      include_last, kv_layout, page_table, page_size)
+                      include_last, kv_layout, page_table, page_size, window_form)
         if return_lse:
             return out[0][..., :D0].contiguous(), out[1]
         return out[..., :D0].contiguous()
@@ -490,18 +517,20 @@ def _decode(q, k, v, cu_seq_lens, seq_lens, scale, max_seq_len, split_tokens, re
         raise ValueError("kv_layout must be 'batched', 'packed' or 'paged'")
     a.max_seqlen = int(bound if max_seq_len is None else min(max_seq_len, bound))
     a.scale_log2 = float(scale) * LOG2E
-    if block_idx is None:
+    gslices = (Hq // Hkv + 31) // 32   # wavefronts per (chunk, kv-head): 32 query heads each
+    if block_idx is None and not window_form:
         a.split_tokens = int(split_tokens) if split_tokens else lib.mi_decode_choose_split_tokens(
-            B, Hkv, a.max_seqlen, _num_cus(lib))
+            B, Hkv * gslices, a.max_seqlen, _num_cus(lib))
     else:
         a.split_tokens = 64
+        a.window_form = 1 if window_form else 0
         a.block_idx, a.block_cnt = _ptr(block_idx), _ptr(block_cnt)
         a.block_idx_stride_b, a.block_idx_stride_h = bi_strides
         a.window_local, a.window_global = window
-        a.include_last_block = 1 if include_last else 0
+        a.include_last_block = 1 if (include_last and not window_form) else 0
         a.max_blocks, a.block_size = int(max_blocks), _masks.BLOCK
         a.split_blocks = int(split_blocks) if split_blocks else lib.mi_decode_choose_split_blocks(
-            B, Hkv, a.max_blocks + a.include_last_block, _num_cus(lib))
+            B, Hkv * gslices, a.max_blocks + a.include_last_block, _num_cus(lib))
     nbytes = lib.mi_decode_workspace_bytes(C.byref(a))
     if nbytes == 0:
         raise _lib.MiAttnError(lib.mi_decode_validate(C.byref(a)), lib.mi_last_error().decode())
@@ -546,7 +575,8 @@ def flash_attention_sparse_decoding(q, k, v, cu_seq_lens, global_window_size=64,
     flash_attn_triton/flash_attn_decoding_sparse.py:222-365: attends the first
     `global_window_size` tokens and the last `local_window_size` tokens of each
     sequence (oracle :391-396); global_window_size must be 64, 128 or 256
-    (:249-253); scale is D^-0.5 (:246).
+    (:249-253); scale is D^-0.5 (:246).  The call is two kernel launches: the
+    blocks a sequence attends are derived from its length inside the kernel.
     Block form — `block_indices` [B,Hkv,n] int32 (unique, ascending, each in
     [0, ceil(len/64))) lists the 64-token blocks each kv-head attends, shared
     by its query heads; `block_counts` [B,Hkv] optionally gives the number of
@@ -564,32 +594,20 @@ def flash_attention_sparse_decoding(q, k, v, cu_seq_lens, global_window_size=64,
         raise ValueError("block_size must be %d" % _masks.BLOCK)
     B, Hq, D = q.shape
     Hkv = k.shape[2]
-    lens = seq_lens if seq_lens is not None else (cu_seq_lens[1:] - cu_seq_lens[:-1])
-    lens = lens.to(torch.int32)
     scale = D ** -0.5
     if block_indices is None:
         gw, lw = int(global_window_size), int(local_window_size)
         assert gw in {64, 128, 256}, "global_window_size must be one of 64, 128, or 256, got %d" % gw
         if lw < 0:
             raise ValueError("local_window_size must be >= 0")
-        n_sink = gw // _masks.BLOCK
-        n_tail = (lw + _masks.BLOCK - 1) // _masks.BLOCK + 1
-        nblk = (lens + _masks.BLOCK - 1) // _masks.BLOCK                      # [B]
-        tail0 = torch.clamp(lens - lw, min=0) // _masks.BLOCK
-        tail0 = torch.maximum(tail0, torch.full_like(tail0, n_sink))           # sink blocks listed once
-        cand = torch.cat([
-            torch.arange(n_sink, device=q.device, dtype=torch.int32).expand(B, n_sink),
-            tail0[:, None] + torch.arange(n_tail, device=q.device, dtype=torch.int32)[None, :],
-        ], dim=1)                                                              # [B, cap]
-        valid = cand < nblk[:, None]
-        key = torch.where(valid, cand, torch.full_like(cand, 2 ** 30))
-        idx = torch.sort(key, dim=1).values.to(torch.int32).contiguous()
-        idx = torch.where(idx >= 2 ** 30, torch.zeros_like(idx), idx)
-        cnt = valid.sum(1).to(torch.int32)[:, None].expand(B, Hkv).contiguous()
-        cap = n_sink + n_tail
-        return _decode(q, k, v, None, lens, scale, None, None, return_lse, block_idx=idx, block_cnt=cnt,
-                       bi_strides=(cap, 0), max_blocks=cap,
-                       split_blocks=split_blocks or 0, window=(lw, gw), **layout)
+        # The blocks a sequence attends follow from (length, gw, lw) alone - the
+        # first gw // 64 blocks, then the blocks from token len - lw to the last -
+        # and the kernel derives them per sequence: no list is built here.
+        cap = gw // _masks.BLOCK + (lw + _masks.BLOCK - 1) // _masks.BLOCK + 1
+        return _decode(q, k, v, cu_seq_lens, seq_lens, scale, None, None, return_lse, max_blocks=cap,
+                       split_blocks=split_blocks or 0, window=(lw, gw), window_form=True, **layout)
+    lens = seq_lens if seq_lens is not None else (cu_seq_lens[1:] - cu_seq_lens[:-1])
+    lens = lens.to(torch.int32)
     if block_indices.dim() != 3 or block_indices.shape[0] != B or block_indices.shape[1] != Hkv \
             or block_indices.is_floating_point():
         raise ValueError("block_indices must be an integer tensor [B, Hkv, n], got %s %s"
