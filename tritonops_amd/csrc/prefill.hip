@@ -186,6 +186,33 @@ struct TileDma {
     else
       asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(koff[t]), "s"(d.kt), "s"(d.sK + inst * 1024) : "memory");
   }
+  // Contiguous rows (pitch = ROWB, e.g. a [B,H,S,D] tensor): the slabs of a
+  // tile are then 1 KiB apart in memory exactly as they are in LDS, and a
+  // load's immediate offset moves both addresses.  M0 is written once per
+  // tensor and tile (pointing kFastMid bytes into the wave's first slab, so
+  // that the offsets of all IPW loads fit the signed 13-bit immediate); loads
+  // t and t + 2 land 16 rows apart, where the swizzle repeats, and share one
+  // lane offset (kfast / vfast).  Load k of 2*IPW: the K loads first, then V.
+  static constexpr int kFastMid = NW * 1024 * (IPW - 1) / 2;
+  static constexpr bool kFastOk = D == 128 && IPW == 4 && NW == 2;
+  uint32_t kfast[2], vfast[2];
+  template <int K>
+  __device__ __forceinline__ void one_fast(const Drip& d) const {
+    constexpr int t = K % IPW;
+    constexpr int imm = NW * 1024 * t - kFastMid;
+    static_assert(imm >= -4096 && imm <= 4095, "immediate offset of a global load");
+    if constexpr (K < IPW) {
+      if constexpr (t == 0)
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3" : : "v"(kfast[t & 1]), "s"(d.kt), "s"(d.sK + wave * 1024 + kFastMid), "n"(imm) : "memory");
+      else
+        asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(kfast[t & 1]), "s"(d.kt), "n"(imm) : "memory");
+    } else {
+      if constexpr (t == 0)
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3" : : "v"(vfast[t & 1]), "s"(d.vt), "s"(d.sV + wave * 1024 + kFastMid), "n"(imm) : "memory");
+      else
+        asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(vfast[t & 1]), "s"(d.vt), "n"(imm) : "memory");
+    }
+  }
   __device__ __forceinline__ void one(const Drip& d, int k) const {
     const int t = k >> 1;
     const int inst = wave + NW * t;
@@ -222,7 +249,16 @@ struct TileDma {
       koff[t] = (uint32_t)r * k_pitch + (uint32_t)(dslot ^ F::swz_k(r)) * 16u;
       voff[t] = (uint32_t)r * v_pitch + (uint32_t)(dslot ^ F::swz_v(r)) * 16u;
     }
+    if constexpr (kFastOk) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        kfast[t] = koff[t] + (uint32_t)(kFastMid - NW * 1024 * t);
+        vfast[t] = voff[t] + (uint32_t)(kFastMid - NW * 1024 * t);
+      }
+    }
   }
+  // do the rows of K and of V follow one another without a gap?
+  __device__ __forceinline__ bool rows_contiguous() const { return k_pitch == F::ROWB && v_pitch == F::ROWB; }
 
   static __device__ __forceinline__ KvSrc<T> source(const T* kp, const T* vp, int len) {
     KvSrc<T> s;
@@ -463,8 +499,10 @@ sparse_kernel(const PrefillParams p) {
   bool hasN = false;
   auto position = [&](auto j_c, auto last_c, auto steady_c, int h) __attribute__((always_inline)) {
     constexpr int J = decltype(j_c)::value;  // h % 2
-    // both requested tiles exist and lie inside the sequence: loads without a mask
+    // both requested tiles exist and lie inside the sequence: loads without a mask;
+    // level 2: rows are contiguous as well, M0 is written once per tensor (TileDma::one_fast)
     constexpr bool STEADY = decltype(steady_c)::value != 0 && D != 96;
+    constexpr bool FAST = decltype(steady_c)::value == 2 && DMA::kFastOk;
     constexpr bool LAST = decltype(last_c)::value != 0;  // no tile h+1: only the second half of block A's arithmetic and block B's MFMAs
     constexpr uint32_t KOFF = (J ^ 1) * TILEB, VOFF = J * TILEB;  // K of tile h+1, V of tile h
     f32x16& Sc = S[J];
@@ -532,12 +570,24 @@ sparse_kernel(const PrefillParams p) {
       }
       if (c >= 8 - G::NDB) vf[c - (8 - G::NDB)] = fr.load_v(VOFF, 0, c - (8 - G::NDB));
       if (!LAST) {
+        if constexpr (FAST) {
+          static_assert(2 * IPW == 8, "one load per MFMA slice");
+          if (c == 0) dma.template one_fast<0>(dK);
+          if (c == 1) dma.template one_fast<1>(dK);
+          if (c == 2) dma.template one_fast<2>(dK);
+          if (c == 3) dma.template one_fast<3>(dK);
+          if (c == 4) dma.template one_fast<4>(dV);
+          if (c == 5) dma.template one_fast<5>(dV);
+          if (c == 6) dma.template one_fast<6>(dV);
+          if (c == 7) dma.template one_fast<7>(dV);
+        } else {
 #pragma unroll
-        for (int k = c * 2 * IPW / 8; k < (c + 1) * 2 * IPW / 8; ++k) {
-          if constexpr (STEADY)
-            dma.one_on((k & 1) ? dV : dK, k);
-          else
-            dma.one((k & 1) ? dV : dK, k);
+          for (int k = c * 2 * IPW / 8; k < (c + 1) * 2 * IPW / 8; ++k) {
+            if constexpr (STEADY)
+              dma.one_on((k & 1) ? dV : dK, k);
+            else
+              dma.one((k & 1) ? dV : dK, k);
+          }
         }
       }
       if (c < 6) {
@@ -606,7 +656,13 @@ sparse_kernel(const PrefillParams p) {
     }
     __syncthreads();  // position 0 requests K(2) into the stage of K(0), which the other wave may still be reading
     int h = 0;
-    if (all_inside) {
+    if (all_inside && DMA::kFastOk && dma.rows_contiguous()) {
+      // ... and the rows of K and V are contiguous: one M0 write per tensor and tile
+      for (; h + 2 < n_tiles; h += 2) {
+        position(ic<0>{}, ic<0>{}, ic<2>{}, h);
+        position(ic<1>{}, ic<0>{}, ic<2>{}, h + 1);
+      }
+    } else if (all_inside) {
       // every listed block lies inside the sequence: the loop whose loads carry no mask
       for (; h + 2 < n_tiles; h += 2) {
         position(ic<0>{}, ic<0>{}, ic<1>{}, h);
