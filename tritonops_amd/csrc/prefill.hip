@@ -859,6 +859,40 @@ dense_kernel(const PrefillParams p) {
     rs = i == 0 ? e_p0 + p1 : rs + (e_p0 + p1);  // pair 0 opens the row sum of its half
     Pd[i] = Elem<T>::pack2(e_p0, p1);
   };
+  // The same work for four pairs (i0 .. i0 + 3) spread over the eight slices of
+  // a block as a pipeline in which no instruction uses the result of its
+  // predecessor: the scaled exponents of a pair are formed a slice before its
+  // exponentials, and its sum and packed pair a slice after them.
+  float su0[2], su1[2], sp0[2], sp1[2], st;
+  auto soft_slice = [&](int c, const f32x16& Sx, int i0, uint32_t (&Pd)[8], float& rs, float mn) __attribute__((always_inline)) {
+    const int j = (c + 1) / 2;      // pair whose exponents are formed in an odd slice / whose first exponential runs in an even one
+    if (c == 0) {
+      su0[0] = fmaf(Sx[2 * i0], scale, mn);
+      su1[0] = fmaf(Sx[2 * i0 + 1], scale, mn);
+      sp0[0] = fast_exp2(su0[0]);
+      return;
+    }
+    if (c & 1) {
+      // odd slice: second exponential of pair (c - 1) / 2, row sum of the pair before it, exponents of the next pair
+      const int k = (c - 1) / 2, sl = k & 1;
+      sp1[sl] = fast_exp2(su1[sl]);
+      if (k > 0) rs = (i0 == 0 && k == 1) ? st : rs + st;
+      if (k < 3) {
+        su0[sl ^ 1] = fmaf(Sx[2 * (i0 + k + 1)], scale, mn);
+        su1[sl ^ 1] = fmaf(Sx[2 * (i0 + k + 1) + 1], scale, mn);
+      } else {
+        const float t2 = sp0[sl] + sp1[sl];
+        Pd[i0 + 3] = Elem<T>::pack2(sp0[sl], sp1[sl]);
+        rs += t2;
+      }
+    } else {
+      // even slice c = 2 j: first exponential of pair j, sum and packed pair of pair j - 1
+      const int sl = j & 1;
+      sp0[sl] = fast_exp2(su0[sl]);
+      st = sp0[sl ^ 1] + sp1[sl ^ 1];
+      Pd[i0 + j - 1] = Elem<T>::pack2(sp0[sl ^ 1], sp1[sl ^ 1]);
+    }
+  };
   // rare: bring m to the exact running maximum including the half in Sx,
   // rescale l and O, and redo the probabilities of that half
   auto exact_fix = [&](const f32x16& Sx, uint32_t (&Pd)[8], float& rs) __attribute__((always_inline)) {
@@ -918,10 +952,7 @@ dense_kernel(const PrefillParams p) {
         if (c + KR < G::KSTEPS) kf[c % KR] = fr.load_k(KOFF, KB ^ 1, c + KR);
       }
       if (c >= 8 - G::NDB) vf[c - (8 - G::NDB)] = fr.load_v(VOFF, 2 * KB, c - (8 - G::NDB));
-      if ((c & 1) == 0)
-        exp_first(Sc, 4 + c / 2, m_neg);
-      else
-        exp_second(4 + c / 2, Pc, rsv[KB]);
+      soft_slice(c, Sc, 4, Pc, rsv[KB], m_neg);
       __builtin_amdgcn_sched_barrier(0);
     }
     // keep the exponentials in this block (they would otherwise sink below
@@ -941,10 +972,7 @@ dense_kernel(const PrefillParams p) {
       }
       if (sl >= 4 && sl - 4 < KR) kf[sl - 4] = fr.load_k(K2OFF, KB, sl - 4);
       // (for the last half of a wave Sn holds scores of stale LDS contents: the results are never used)
-      if ((sl & 1) == 0)
-        exp_first(Sn, sl / 2, m_neg);
-      else
-        exp_second(sl / 2, Pn, rsv[KB ^ 1]);
+      soft_slice(sl, Sn, 0, Pn, rsv[KB ^ 1], m_neg);
       __builtin_amdgcn_sched_barrier(0);
     }
     asm volatile("" : "+v"(Pn[0]), "+v"(Pn[1]), "+v"(Pn[2]), "+v"(Pn[3]), "+v"(rsv[KB ^ 1]));
