@@ -46,18 +46,43 @@ def _regs(line):
     return found
 
 
+def _significant(lines):
+    """(index, text) of the instruction lines: no comments, directives or labels."""
+    out = []
+    for i, l in enumerate(lines):
+        t = l.split(";")[0].strip()
+        if t and not t.startswith(".") and not t.endswith(":"):
+            out.append((i, t))
+    return out
+
+
 def test_output_store_count_matches_the_counted_wait(dense_kernels):
     # At an item boundary a wave issues: Q and tile 0, the first half of its
     # output stores, tile 1, the second half of the stores, tile 2.  The wait at
     # the top of the next item leaves that second half and the loads of tile 2
-    # in flight: half the stores plus the loads of one tile per wave.
+    # in flight: half the stores plus the loads of one tile per wave.  That wait
+    # is the one site in the kernel where a counted wait and a full wait are the
+    # two arms of one decision (all stores issued or not), joined in front of
+    # the barrier that opens the item with no vector-memory instruction between.
     for (dtype, d), lines in dense_kernels.items():
         stores = [l for l in lines if "global_store_dwordx4" in l]
         expect = {64: 4, 96: 8, 128: 8}[d]
         assert len(stores) == expect, (dtype, d, len(stores))
         tile_loads = {64: 2, 96: 4, 128: 4}[d]      # K and V instructions of one tile per wave
-        waits = {int(x) for l in lines for x in re.findall(r"^\s*s_waitcnt vmcnt\((\d+)\)\s*$", l)}
-        assert expect // 2 + tile_loads in waits, (dtype, d, waits)
+        want = expect // 2 + tile_loads
+        sig = _significant(lines)
+        sites = []
+        for k, (_, t) in enumerate(sig):
+            if t != "s_waitcnt vmcnt(%d)" % want:
+                continue
+            arm = [x for _, x in sig[k + 1:k + 4]]
+            if "s_waitcnt vmcnt(0)" not in arm:
+                continue                                  # some other wait that happens to have the same count
+            j = k + 1 + arm.index("s_waitcnt vmcnt(0)")
+            nxt = next(x for _, x in sig[j + 1:] if x.startswith("s_barrier") or re.match(r"(global|buffer|scratch|flat)_", x))
+            assert nxt.startswith("s_barrier"), (dtype, d, nxt)
+            sites.append(k)
+        assert len(sites) == 1, (dtype, d, want, sites)
 
 
 def test_no_scratch_memory(dense_kernels):
