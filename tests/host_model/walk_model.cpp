@@ -15,6 +15,9 @@
 //     wait covers its loads) and published by a barrier; no stage is written in
 //     a barrier interval in which a wave reads it; the Q registers have landed
 //     before their first use.
+//   block-sparse forward (prefill.hip, sparse_kernel): the two-stage K ring that
+//     runs one tile ahead of the two-stage V ring; the block list held in two
+//     64-entry registers; every tile read is the tile of the listed block.
 //   softmax with a running reference point (no row maximum in the common
 //     path): equals the plain softmax, also for scores that keep growing.
 //   decode (decode.hip): the window form's arithmetic block list equals the
@@ -32,7 +35,7 @@
 #include <vector>
 
 static int g_fail = 0;
-// 0: the kernels' protocols as they are.  1..8: one deliberate mistake each; the
+// 0: the kernels' protocols as they are.  1..10: one deliberate mistake each; the
 // run must then fail (tests/test_host_model.py checks that it does), which is
 // what shows that the checks below can tell a broken protocol from a sound one.
 static int g_mut = 0;
@@ -367,6 +370,123 @@ static void test(std::mt19937& rng) {
 }
 }  // namespace dense
 
+// ------------------------------------------------------------------ block-sparse
+namespace sparse {
+// prefill.hip, sparse_kernel: two wavefronts walk the tiles of a CSR row (a
+// listed 64-key block is two 32-key tiles).  K tiles run one position ahead of
+// V tiles and each tensor has a ring of two stages; the block list is held 64
+// entries at a time in two registers and read with a lane index.
+constexpr int NW = 2;
+struct Stage {
+  int tile = -1, block = -1, issued_in = -1;
+  bool landed[NW] = {}, published = false;
+};
+struct Machine {
+  Stage k[2], v[2];
+  int interval = 0;
+  std::vector<const Stage*> read_now;
+  std::vector<std::pair<Stage*, int>> in_flight[NW];  // (stage, tile) per wave, in issue order
+  void request(int w, Stage& s, int tile, int block) {
+    if (s.tile != tile || s.issued_in != interval) {
+      s.tile = tile; s.block = block; s.issued_in = interval; s.published = false;
+      for (bool& l : s.landed) l = false;
+    }
+    for (const Stage* r : read_now) CHECK(r != &s, "tile %d is requested into a stage that is read in the same barrier interval", tile);
+    in_flight[w].push_back({&s, tile});
+  }
+  void wait_all(int w) {
+    for (auto& f : in_flight[w])
+      if (f.first->tile == f.second) f.first->landed[w] = true;
+    in_flight[w].clear();
+  }
+  void read(int w, const Stage& s, int tile, int block, const char* what) {
+    CHECK(s.tile == tile && s.block == block, "wave %d reads %s of tile %d (block %d), the stage holds tile %d (block %d)", w, what, tile, block, s.tile, s.block);
+    CHECK(s.published && s.issued_in < interval, "wave %d reads %s of tile %d before it is published", w, what, tile);
+    read_now.push_back(&s);
+  }
+  void barrier() {
+    ++interval;
+    read_now.clear();
+    for (Stage* s : {&k[0], &k[1], &v[0], &v[1]})
+      if (s->tile >= 0 && s->landed[0] && s->landed[1]) s->published = true;
+  }
+};
+
+static void walk(const std::vector<int>& cols) {
+  const int n_blk = (int)cols.size(), n_tiles = 2 * n_blk;
+  if (n_tiles == 0) return;
+  Machine m;
+  // the list registers of a wave: entry 64 * chunk + lane, the chunk walked and the one behind it
+  auto load_cols = [&](int chunk) {
+    std::vector<int> r(64, 0);
+    for (int l = 0; l < 64; ++l)
+      if (chunk * 64 + l < n_blk) r[l] = cols[chunk * 64 + l];
+    return r;
+  };
+  struct WaveRegs {
+    int col_chunk = 0;
+    std::vector<int> col_cur, col_nxt;
+    int blkC = 0, blkN = 0;
+    bool hasN = false;
+  } wr[NW];
+  for (auto& r : wr) { r.col_cur = load_cols(0); r.col_nxt = load_cols(1); }
+  // prologue: K and V of tile 0, K of tile 1; full wait; barrier; scores of tile 0; barrier
+  for (int w = 0; w < NW; ++w) {
+    wr[w].blkC = wr[w].col_cur[0];
+    m.request(w, m.k[0], 0, wr[w].blkC);
+    m.request(w, m.v[0], 0, wr[w].blkC);
+    m.request(w, m.k[1], 1, wr[w].blkC);
+    m.wait_all(w);
+  }
+  m.barrier();
+  for (int w = 0; w < NW; ++w) m.read(w, m.k[0], 0, cols[0], "K");
+  if (g_mut != 9) m.barrier();
+  for (int h = 0; h < n_tiles; ++h) {
+    const int J = h & 1;
+    const bool last = h == n_tiles - 1;
+    for (int w = 0; w < NW; ++w) {
+      WaveRegs& r = wr[w];
+      if (J == 0) {
+        const int bn = (h >> 1) + 1;
+        r.hasN = bn < n_blk;
+        if (r.hasN) {
+          if ((bn >> 6) != r.col_chunk) {
+            ++r.col_chunk;
+            r.col_cur = r.col_nxt;
+            r.col_nxt = load_cols(r.col_chunk + (g_mut == 10 ? 0 : 1));
+          }
+          r.blkN = r.col_cur[bn & 63];
+        }
+      }
+      const bool has1 = J == 0 ? true : r.hasN, has2 = r.hasN;
+      if (!last) {
+        // K of tile h + 2 into the K stage of tile h, V of tile h + 1 into the V stage of tile h - 1
+        if (has2) m.request(w, m.k[J], h + 2, r.blkN);
+        if (has1) m.request(w, m.v[J ^ 1], h + 1, J == 0 ? r.blkC : r.blkN);
+        m.read(w, m.k[J ^ 1], h + 1, cols[(h + 1) >> 1], "K");
+      }
+      m.read(w, m.v[J], h, cols[h >> 1], "V");
+      if (!last) {
+        if (J == 1) r.blkC = r.blkN;
+        m.wait_all(w);
+      }
+    }
+    if (!last) m.barrier();
+  }
+}
+
+static void test(std::mt19937& rng) {
+  int cases = 0;
+  for (int n = 0; n <= 400; ++n) {
+    std::vector<int> cols(n);
+    for (auto& c : cols) c = (int)(rng() % 100000);   // any block ids: the walk must name them in list order
+    walk(cols);
+    ++cases;
+  }
+  std::printf("block-sparse walk: %d lists\n", cases);
+}
+}  // namespace sparse
+
 // ------------------------------------------------------------------ softmax
 namespace softmax {
 // prefill.hip: probabilities of a half (16 scores per lane of a row here: the
@@ -519,6 +639,7 @@ int main(int argc, char** argv) {
   if (argc > 1) g_mut = std::atoi(argv[1]);
   std::mt19937 rng(12345);
   if (g_mut != 5 && g_mut != 6) dense::test(rng);   // (those two mistakes sit in the other parts)
+  sparse::test(rng);
   softmax::test(rng);
   decode::test(rng);
   if (g_fail) {
