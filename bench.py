@@ -135,9 +135,14 @@ def _fwd_args(q, k, v, o, lse, causal):
     return a
 
 
+# (batch, heads, sequence length) of the dense causal workload; --dense-shape replaces it for profiling other
+# shapes (the headline line of the default run is always the benchmark's own configuration)
+DENSE_SHAPE = (4, 32, 8192)
+
+
 def run_dense_causal(steps, warmup):
     import tritonops_amd as ta
-    B, H, S, D = 4, 32, 8192, 128
+    (B, H, S), D = DENSE_SHAPE, 128
     q, k, v = (_randn((B, H, S, D), s) for s in (0, 1, 2))
     fn = lambda: ta.flash_attention(q, k, v, causal=True, return_lse=True)
     ms = _time_steps(fn, steps, warmup)
@@ -148,8 +153,8 @@ def run_dense_causal(steps, warmup):
     # parity on the benchmark tensors: three (batch, head) units x four 64-row blocks
     err = err_lse = 0.0
     keys = torch.arange(S, device="cuda")
-    for b, h in ((0, 0), (1, 13), (3, 31)):
-        for r0 in (0, 1984, 4096, S - 64):
+    for b, h in ((0, 0), (min(1, B - 1), 13 % H), (B - 1, H - 1)):
+        for r0 in sorted({0, (S // 4 - 64) // 64 * 64, S // 2, S - 64}):
             rows = torch.arange(r0, r0 + 64, device="cuda")
             want, want_lse = _ref_rows(q[b, h], k[b, h], v[b, h], rows, D ** -0.5, keys[None, :] <= rows[:, None])
             err = max(err, _err(o[b, h, rows], want))
@@ -161,7 +166,7 @@ def run_dense_causal(steps, warmup):
         "err_sample": "o and lse of 3 (batch, head) units x 4 blocks of 64 query rows against fp32 torch math on the device",
         "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "kernel": KERNELS["dense_causal"]},
-        "config": {"workload": "dense causal flash-attention fwd bf16 B=4 H=32 S=8192 D=128, o bf16 + lse fp32",
+        "config": {"workload": "dense causal flash-attention fwd bf16 B=%d H=%d S=%d D=128, o bf16 + lse fp32" % (B, H, S),
                    "flop_per_step": flop, "flop_reference_convention_4BHS2D": 4.0 * B * H * S * S * D},
     }
 
@@ -978,7 +983,15 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also launch one elementwise copy of 1 GiB (2 GiB of HBM traffic) as the reference "
                          "dispatch for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
+    ap.add_argument("--dense-shape", default=None, metavar="B,H,S",
+                    help="batch, heads and sequence length of the dense_causal workload instead of the benchmark's "
+                         "4,32,8192 (S a multiple of 64, at least 256; for profiling other shapes)")
     a = ap.parse_args()
+    if a.dense_shape:
+        global DENSE_SHAPE
+        DENSE_SHAPE = tuple(int(x) for x in a.dense_shape.split(","))
+        if len(DENSE_SHAPE) != 3 or min(DENSE_SHAPE) < 1 or DENSE_SHAPE[2] % 64 or DENSE_SHAPE[2] < 256:
+            sys.exit("bench.py: --dense-shape takes B,H,S with S a multiple of 64, at least 256")
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the attention path shards over batch and "
                  "heads without communication); run with --gpus 1")

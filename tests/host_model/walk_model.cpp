@@ -65,7 +65,7 @@ struct Geo {
 };
 
 // prefill.hip: item_geo
-static bool item_geo(const Shape& s, int n_qtiles, int bid, Geo& g) {
+static bool item_geo(const Shape& s, int n_qtiles, int bid, Geo& g, int bm = BM) {
   const int gqa = s.hq / s.hkv;
   const int per_unit = n_qtiles * gqa;
   const int n_units = s.batch * s.hkv;
@@ -83,7 +83,7 @@ static bool item_geo(const Shape& s, int n_qtiles, int bid, Geo& g) {
   g.kvh = unit % s.hkv;
   g.h = g.kvh * gqa + r % gqa;
   g.len = std::min(s.lens[g.b], s.max_seqlen);
-  return g.qt * BM < g.len;
+  return g.qt * bm < g.len;
 }
 
 // One vector-memory operation of a wave, in issue order.
@@ -92,11 +92,12 @@ struct VmOp {
   int item, tile;  // TILE: which tile of which item
 };
 
-struct Stage {
+template <int NWAVES>
+struct StageT {
   int item = -1, tile = -1;   // latest request
   int issued_in = -1;         // barrier interval of the latest request
-  bool landed[NW] = {};       // wave w's loads of it have retired
-  bool published = false;     // a barrier has passed since all eight landed
+  bool landed[NWAVES] = {};   // wave w's loads of it have retired
+  bool published = false;     // a barrier has passed since all of them landed
 };
 
 struct Wave {
@@ -105,9 +106,11 @@ struct Wave {
   int q_item = -1;
 };
 
-struct Machine {
-  Stage st[NS];
-  Wave wv[NW];
+template <int NWAVES, int NSTAGES>
+struct MachineT {
+  using Stage = StageT<NWAVES>;
+  Stage st[NSTAGES];
+  Wave wv[NWAVES];
   int interval = 0;                 // barriers passed so far
   std::vector<std::pair<int, int>> reads_this_interval;  // (stage, wave)
   int ipw2;                         // loads per tile and wave (K + V)
@@ -162,6 +165,8 @@ struct Machine {
   }
 };
 
+using Machine = MachineT<NW, NS>;
+
 struct Item {
   int id, len, q0, n_tiles;
 };
@@ -174,6 +179,52 @@ struct Step {
   int a = 0, b = 0, c = 0;  // WAIT: n; REQ_TILE: stage, item, tile; READ: stage, item, tile; STORE: count
   const char* what = "";
 };
+
+// Runs the per-wave programs barrier interval by barrier interval: inside an
+// interval the waves are independent, so wave 0, 1, ... each run up to their
+// next barrier, then the barrier happens for all of them.
+template <class M>
+static void execute(std::vector<std::vector<Step>>& prog, M& m, int ksteps) {
+  const int nw = (int)prog.size();
+  std::vector<size_t> pc(nw, 0);
+  for (;;) {
+    int at_barrier = 0, done = 0;
+    for (int w = 0; w < nw; ++w) {
+      auto& P = prog[w];
+      while (pc[w] < P.size() && P[pc[w]].kind != Step::BARRIER) {
+        const Step& st = P[pc[w]++];
+        switch (st.kind) {
+          case Step::WAIT: m.wait(w, st.a); break;
+          case Step::REQ_Q:
+            m.wv[w].q_item = st.a;
+            m.wv[w].q_landed = false;
+            for (int i = 0; i < ksteps; ++i) m.wv[w].vm.push_back({VmOp::Q, st.a, 0});
+            break;
+          case Step::USE_Q:
+            CHECK(m.wv[w].q_item == st.a && m.wv[w].q_landed, "wave %d uses the Q registers of item %d before its loads have retired", w, st.a);
+            break;
+          case Step::REQ_TILE: m.request_tile(w, st.a, st.b, st.c); break;
+          case Step::READ: m.read(w, st.a, st.b, st.c, st.what); break;
+          case Step::STORE:
+            for (int i = 0; i < st.a; ++i) m.wv[w].vm.push_back({VmOp::STORE, 0, 0});
+            break;
+          case Step::STAGE_TOUCH:
+            // the staging area must not be the target of a tile load that is under way
+            CHECK(m.st[st.a].issued_in < m.interval || m.st[st.a].item < 0, "write-out stages through stage %d while a tile is being loaded into it", st.a);
+            m.reads_this_interval.push_back({st.a, w});
+            break;
+          default: break;
+        }
+      }
+      if (pc[w] < P.size()) ++at_barrier; else ++done;
+    }
+    if (done == nw) break;
+    CHECK(at_barrier == nw, "waves disagree on the number of barriers (%d at a barrier, %d finished)", at_barrier, done);
+    if (at_barrier != nw) break;
+    for (int w = 0; w < nw; ++w) ++pc[w];
+    m.barrier();
+  }
+}
 
 static void run(const Shape& s, int grid, int ksteps, int ipw, int out_stores_full, Machine& m,
                 std::vector<int>& visited) {
@@ -288,45 +339,7 @@ static void run(const Shape& s, int grid, int ksteps, int ipw, int out_stores_fu
         if (in_flight_ok) CHECK(live == per_pass, "full rows but %d of %d store instructions", live, per_pass);
       }
     }
-    // ---- run interval by interval
-    std::vector<size_t> pc(NW, 0);
-    for (;;) {
-      int at_barrier = 0, done = 0;
-      for (int w = 0; w < NW; ++w) {
-        auto& P = prog[w];
-        while (pc[w] < P.size() && P[pc[w]].kind != Step::BARRIER) {
-          const Step& st = P[pc[w]++];
-          switch (st.kind) {
-            case Step::WAIT: m.wait(w, st.a); break;
-            case Step::REQ_Q:
-              m.wv[w].q_item = st.a;
-              m.wv[w].q_landed = false;
-              for (int i = 0; i < ksteps; ++i) m.wv[w].vm.push_back({VmOp::Q, st.a, 0});
-              break;
-            case Step::USE_Q:
-              CHECK(m.wv[w].q_item == st.a && m.wv[w].q_landed, "wave %d uses the Q registers of item %d before its loads have retired", w, st.a);
-              break;
-            case Step::REQ_TILE: m.request_tile(w, st.a, st.b, st.c); break;
-            case Step::READ: m.read(w, st.a, st.b, st.c, st.what); break;
-            case Step::STORE:
-              for (int i = 0; i < st.a; ++i) m.wv[w].vm.push_back({VmOp::STORE, 0, 0});
-              break;
-            case Step::STAGE_TOUCH:
-              // the staging area must not be the target of a tile load that is under way
-              CHECK(m.st[st.a].issued_in < m.interval || m.st[st.a].item < 0, "write-out stages through stage %d while a tile is being loaded into it", st.a);
-              m.reads_this_interval.push_back({st.a, w});
-              break;
-            default: break;
-          }
-        }
-        if (pc[w] < P.size()) ++at_barrier; else ++done;
-      }
-      if (done == NW) break;
-      CHECK(at_barrier == NW, "waves disagree on the number of barriers (%d at a barrier, %d finished)", at_barrier, done);
-      if (at_barrier != NW) break;
-      for (int w = 0; w < NW; ++w) ++pc[w];
-      m.barrier();
-    }
+    execute(prog, m, ksteps);
   }
 }
 
