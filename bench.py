@@ -52,6 +52,10 @@ KERNELS = {
         "19rms_dw_stage_kernelILi4EEEvPKfPfii", "20rms_dw_reduce_kernelIfEEvPKfPT_ii")),
     "fused_xent": _NS + "16xent_gemm_kernelIDF16bLb0EEEvNS_10XentParamsE",
 }
+# the reference's own call forms run on the kernels of the configurations above
+KERNELS["dense_causal_packed"] = KERNELS["dense_causal"]
+KERNELS["window_sparse_prefill"] = KERNELS["block_sparse"]
+KERNELS["window_sparse_decode"] = KERNELS["sparse_decode"]
 
 
 def _sync():
@@ -636,7 +640,7 @@ def run_dense_packed(steps, warmup):
         "max_abs_err": max(m["err"], r["err"]), "max_abs_err_lse2": max(m["err_lse"], r["err_lse"]),
         "err_sample": "o and lse of 2 heads x 3 blocks of 64 query rows in 3 sequences of each mix against fp32 torch math on the device",
         "roofline": {"bound": "mfma", "achieved": m["flop"] / (m["kms"] * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "kernel": KERNELS["dense_causal"]},
+                     "unit": "TFLOP/s", "kernel": KERNELS["dense_causal_packed"]},
         "config": {"workload": "dense causal fwd bf16, packed [1,32768,32,128] + cu_seq_lens for 4 x 8192 tokens, through "
                                "flash_attention(q, k, v, cu_seq_lens) with uninitialised outputs (the library zeroes "
                                "rows outside the sequences) and the longest length cached per cu_seq_lens tensor",
@@ -705,7 +709,7 @@ def run_window_sparse_prefill(steps, warmup):
         "max_abs_err": err, "max_abs_err_lse2": err_lse,
         "err_sample": "o and lse of all heads x 4 blocks of 64 query rows in 2 of the 4 sequences against masked fp32 torch math on the device",
         "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "kernel": KERNELS["block_sparse"]},
+                     "unit": "TFLOP/s", "kernel": KERNELS["window_sparse_prefill"]},
         "config": {"workload": "window-sparse causal fwd bf16, packed [1,32768,16,128] + cu_seqlens for 4 x 8192 tokens, local "
                                "window 1024, global window 128, through flash_attn_sparse_triton(q, k, v, cu, None, 1024, 128)",
                    "flop_per_step": flop, "wall_over_kernel": ms / kms,
@@ -767,7 +771,7 @@ def run_window_sparse_decode(steps, warmup):
         "max_abs_err": err,
         "err_sample": "3 of the 32 sequences (all heads) against fp32 torch math over the attended tokens on the device",
         "roofline": {"bound": "hbm", "achieved": nbytes_alg / (k_split * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "kernel": KERNELS["sparse_decode"]},
+                     "unit": "GB/s", "kernel": KERNELS["window_sparse_decode"]},
         "config": {"workload": "window-sparse decode bf16 B=32 Hq=32 Hkv=8 KV=131072 D=128, global window 256 + local window "
                                "4096, through flash_attention_sparse_decoding(q, k, v, cu_seq_lens, 256, 4096): two "
                                "launches, the block list is derived inside the kernel",
