@@ -40,7 +40,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 _NS = "_ZN2mi12_GLOBAL__N_1"
 KERNELS = {
     "dense_causal": _NS + "12dense_kernelIDF16bLi128EEEvNS_13PrefillParamsE",
-    "c1_dense_noncausal_small": _NS + "12dense_kernelIDF16bLi64EEEvNS_13PrefillParamsE",
+    "c1_dense_noncausal_small": _NS + "18dense_short_kernelIDF16bLi64EEEvNS_13PrefillParamsE",
     "gqa_decode": _NS + "21decode_splitkv_kernelIDF16bLi128EEEvNS_12DecodeParamsE",
     "block_sparse": _NS + "13sparse_kernelIDF16bLi128EEEvNS_13PrefillParamsE",
     "sparse_decode": _NS + "21decode_splitkv_kernelIDF16bLi128EEEvNS_12DecodeParamsE",

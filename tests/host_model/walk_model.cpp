@@ -9,7 +9,8 @@
 // shapes; it is built with -fsanitize=address,undefined by
 // tests/test_host_model.py, so that an index that leaves its array fails loudly.
 //
-//   dense forward (prefill.hip, dense_kernel): work-item map and persistent
+//   dense forward (prefill.hip, dense_kernel and its short form
+//     dense_short_kernel): work-item map and persistent
 //     schedule visit every (sequence, head, q tile) once; every LDS stage a wave
 //     reads holds the tile it expects, requested, landed (the wave's counted
 //     wait covers its loads) and published by a barrier; no stage is written in
@@ -35,7 +36,7 @@
 #include <vector>
 
 static int g_fail = 0;
-// 0: the kernels' protocols as they are.  1..10: one deliberate mistake each; the
+// 0: the kernels' protocols as they are.  1..12: one deliberate mistake each; the
 // run must then fail (tests/test_host_model.py checks that it does), which is
 // what shows that the checks below can tell a broken protocol from a sound one.
 static int g_mut = 0;
@@ -343,6 +344,102 @@ static void run(const Shape& s, int grid, int ksteps, int ipw, int out_stores_fu
   }
 }
 
+// prefill.hip, dense_short_kernel: 4 waves, 128 rows per item, tiles of 32 keys
+// in five stages; tile j is requested at the top of position j - 4; at the top
+// of position h tiles up to h + 2 must have landed.
+namespace short_form {
+constexpr int NW = 4, NS = 5, TN = 32, BM = 128;
+using Machine = MachineT<NW, NS>;
+
+static void run(const Shape& s, int grid, int ksteps, int ipw, std::vector<int>& visited) {
+  const int n_qtiles = (s.max_seqlen + BM - 1) / BM;
+  const int n_items = n_qtiles * s.hq * s.batch;
+  for (int wg = 0; wg < grid; ++wg) {
+    std::vector<Item> items;
+    int round = 0;
+    for (int base = 0; base < n_items; base += grid, ++round) {
+      int w = wg;
+      if ((round & 1) && (grid & 7) == 0) w = (((grid >> 3) - 1 - (w >> 3)) << 3) | (w & 7);
+      const int bid = base + w;
+      Geo g;
+      if (bid < n_items) {
+        ++visited[bid];
+        if (item_geo(s, n_qtiles, bid, g, BM)) {
+          Item it;
+          it.id = bid;
+          it.len = g.len;
+          it.q0 = g.qt * BM;
+          it.n_tiles = (g.len + TN - 1) / TN;
+          if (s.causal) it.n_tiles = std::min(it.n_tiles, (it.q0 + BM + TN - 1) / TN);
+          items.push_back(it);
+        }
+      }
+    }
+    if (items.empty()) continue;
+    Machine m;
+    m.ipw2 = 2 * ipw;
+    std::vector<std::vector<Step>> prog(NW);
+    for (int w = 0; w < NW; ++w) {
+      auto& P = prog[w];
+      auto req_tile = [&](int stage, const Item& it, int t) {
+        if (t < it.n_tiles) P.push_back({Step::REQ_TILE, stage, it.id, t});
+      };
+      P.push_back({Step::REQ_Q, items[0].id});
+      for (int t = 0; t < NS - 1; ++t) req_tile(t, items[0], t);
+      for (size_t k = 0; k < items.size(); ++k) {
+        const Item& it = items[k];
+        const int q0w = it.q0 + 32 * w;
+        int H_w = (it.len + 31) / 32;
+        if (s.causal) H_w = std::min(H_w, q0w / 32 + 1);
+        H_w = std::min(H_w, it.n_tiles);
+        if (q0w >= it.len) H_w = 0;
+        const int tail_h = std::max(1, it.n_tiles - (NS - 1));
+        // item top: tile 3, when it exists, is the youngest request and may stay in flight
+        int allow = (NS - 2 < it.n_tiles) ? 2 * ipw : 0;
+        if (g_mut == 11) allow = 2 * ipw;
+        P.push_back({Step::WAIT, allow});
+        P.push_back({Step::USE_Q, it.id});
+        P.push_back({Step::BARRIER});
+        req_tile(NS - 1, it, NS - 1);
+        if (H_w > 0) P.push_back({Step::READ, 0, it.id, 0, "K of tile 0"});
+        for (int h = 0; h < it.n_tiles; ++h) {
+          if (h > 0) {
+            if (h + NS - 1 < it.n_tiles) {
+              P.push_back({Step::WAIT, (g_mut == 12 ? NS - 3 : NS - 4) * 2 * ipw});
+              P.push_back({Step::BARRIER});
+              req_tile((h + NS - 1) % NS, it, h + NS - 1);
+            } else if (h == tail_h) {
+              P.push_back({Step::WAIT, 0});
+              P.push_back({Step::BARRIER});
+            }
+          }
+          if (h >= H_w) continue;
+          if (h + 1 < H_w) P.push_back({Step::READ, (h + 1) % NS, it.id, h + 1, "K of the next tile"});
+          P.push_back({Step::READ, h % NS, it.id, h, "V"});
+          if (h + 2 < H_w) P.push_back({Step::READ, (h + 2) % NS, it.id, h + 2, "first K fragments two tiles ahead"});
+        }
+        P.push_back({Step::BARRIER});
+        const bool more = k + 1 < items.size();
+        if (more) {
+          P.push_back({Step::REQ_Q, items[k + 1].id});
+          req_tile(0, items[k + 1], 0);
+        }
+        const int rows = std::max(0, std::min(32, it.len - q0w));
+        P.push_back({Step::STAGE_TOUCH, NS - 1});
+        P.push_back({Step::STORE, rows > 0 ? 2 : 0});
+        if (more) req_tile(1, items[k + 1], 1);
+        P.push_back({Step::STORE, rows > 0 ? 2 : 0});
+        if (more) {
+          req_tile(2, items[k + 1], 2);
+          req_tile(3, items[k + 1], 3);
+        }
+      }
+    }
+    execute(prog, m, ksteps);
+  }
+}
+}  // namespace short_form
+
 static void test(std::mt19937& rng) {
   int cases = 0;
   for (int rep = 0; rep < 200; ++rep) {
@@ -366,6 +463,20 @@ static void test(std::mt19937& rng) {
         run(s, grid, ksteps, ipw, out_stores, m, visited);
         for (int i = 0; i < n_items; ++i) CHECK(visited[i] == 1, "work item %d of %d visited %d times (grid %d)", i, n_items, visited[i], grid);
         ++cases;
+      }
+    }
+    // the short form of the same kernel (head_dim 64): 128-row items, three workgroups per CU
+    {
+      const int nq = (s.max_seqlen + short_form::BM - 1) / short_form::BM;
+      const int ni = nq * s.hq * s.batch;
+      for (int grid : {1, 5, 16, 768}) {
+        if (grid > ni) grid = ni;
+        for (int d : {64, 128}) {   // (128: two tile loads per wave and tensor instead of one; the kernel is generic)
+          std::vector<int> visited(ni, 0);
+          short_form::run(s, grid, d / 16, d == 64 ? 1 : 2, visited);
+          for (int i = 0; i < ni; ++i) CHECK(visited[i] == 1, "short form: work item %d of %d visited %d times (grid %d)", i, ni, visited[i], grid);
+          ++cases;
+        }
       }
     }
     // the item map is a bijection onto (sequence, q head, q tile)

@@ -2,7 +2,7 @@
 AddressSanitizer and UndefinedBehaviorSanitizer and run on the CPU.
 
 The model restates, without any device code, the work-item map and persistent
-schedule of the dense forward kernel, its four-stage tile ring with the counted
+schedule of the dense forward kernel, its four-stage tile ring (and the five-stage ring of its short form) with the counted
 vector-memory waits and barriers, the running-reference softmax, the window
 form's block list and the dealing of decode chunks, and checks their invariants
 over thousands of ragged shapes.  Each of its deliberate-mistake modes breaks one
@@ -28,6 +28,8 @@ MISTAKES = {
     8: "the counted wait is used also behind partial output stores",
     9: "block-sparse: no barrier between the scores of tile 0 and the request of K of tile 2",
     10: "block-sparse: the list register behind the walked one is refilled with the wrong 64 entries",
+    11: "short form: the wait at the top of an item always leaves one tile in flight",
+    12: "short form: the wait at the top of a position leaves two tiles in flight",
 }
 
 

@@ -20,7 +20,7 @@ HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 
 
 @pytest.fixture(scope="module")
-def dense_kernels(tmp_path_factory):
+def prefill_asm(tmp_path_factory):
     if not os.path.exists(HIPCC):
         pytest.skip("hipcc not available")
     out = tmp_path_factory.mktemp("asm") / "prefill.s"
@@ -28,12 +28,28 @@ def dense_kernels(tmp_path_factory):
            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
            "-I", os.path.join(ROOT, "include"), "--cuda-device-only", "-S", SRC, "-o", str(out)]
     subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
-    text = out.read_text()
+    return out.read_text()
+
+
+def _bodies(text, family):
     kernels = {}
-    for m in re.finditer(r"^(_ZN2mi\S*dense_kernelI(\S+?)Li(\d+)E\S*):", text, re.M):
+    for m in re.finditer(r"^(_ZN2mi\S*\d%sI(\S+?)Li(\d+)E\S*):" % family, text, re.M):
         body = text[m.end():text.index("s_endpgm", m.end())]
         kernels[(m.group(2), int(m.group(3)))] = body.split("\n")
+    return kernels
+
+
+@pytest.fixture(scope="module")
+def dense_kernels(prefill_asm):
+    kernels = _bodies(prefill_asm, "dense_kernel")
     assert len(kernels) == 6, sorted(kernels)          # bf16 / f16  x  64 / 96 / 128
+    return kernels
+
+
+@pytest.fixture(scope="module")
+def short_kernels(prefill_asm):
+    kernels = _bodies(prefill_asm, "dense_short_kernel")
+    assert sorted(kernels) == [("DF16_", 64), ("DF16b", 64)], sorted(kernels)   # the short form is built for head_dim 64
     return kernels
 
 
@@ -85,13 +101,43 @@ def test_output_store_count_matches_the_counted_wait(dense_kernels):
         assert len(sites) == 1, (dtype, d, want, sites)
 
 
-def test_no_scratch_memory(dense_kernels):
-    for key, lines in dense_kernels.items():
+def test_no_scratch_memory(dense_kernels, short_kernels):
+    for key, lines in list(dense_kernels.items()) + list(short_kernels.items()):
         assert not any("scratch_" in l for l in lines), key
 
 
-def test_q_registers_are_untouched_between_load_and_wait(dense_kernels):
-    for (dtype, d), lines in dense_kernels.items():
+def test_short_form_leaves_room_for_three_waves_per_simd(prefill_asm, short_kernels):
+    """Three 4-wave workgroups share a CU, one wave of each per SIMD: 512 registers
+    in allocation units of 8 leave 168 per wave.  And the item-top wait: when the
+    next item has a fourth tile its loads (one K and one V instruction per wave at
+    head_dim 64) are the youngest and may stay in flight, else everything is
+    waited for; the two arms meet in front of the barrier that opens the item."""
+    seen = 0
+    for block in prefill_asm.split("- .agpr_count:")[1:]:
+        kern = re.search(r"\.name:\s+(\S+)", block).group(1)
+        if "dense_short_kernel" in kern:
+            assert int(re.search(r"\.vgpr_count:\s+(\d+)", block).group(1)) <= 168, kern
+            seen += 1
+    assert seen == 2
+    for key, lines in short_kernels.items():
+        assert len([l for l in lines if "global_store_dwordx4" in l]) == 4, key
+        sig = _significant(lines)
+        sites = []
+        for k, (_, t) in enumerate(sig):
+            if t != "s_waitcnt vmcnt(2)":
+                continue
+            near = [j for j in range(max(0, k - 5), min(len(sig), k + 6)) if sig[j][1] == "s_waitcnt vmcnt(0)"]
+            if not near:
+                continue                                  # (the waits at the top of a position also cover lgkmcnt)
+            last = max(near + [k])
+            nxt = next(x for _, x in sig[last + 1:] if x.startswith("s_barrier") or re.match(r"(global|buffer|scratch|flat)_", x))
+            assert nxt.startswith("s_barrier"), (key, nxt)
+            sites.append(k)
+        assert len(sites) == 1, (key, sites)
+
+
+def test_q_registers_are_untouched_between_load_and_wait(dense_kernels, short_kernels):
+    for (dtype, d), lines in list(dense_kernels.items()) + list(short_kernels.items()):
         loads = [(i, l) for i, l in enumerate(lines)
                  if re.match(r"\s*global_load_dwordx4 v\[\d+:\d+\], v\[\d+:\d+\], off offset:", l)]
         ksteps = d // 16

@@ -197,6 +197,12 @@ int launch_xent_dlogits(const XentGradParams& p, int dtype, hipStream_t s);
 // Query rows per workgroup of the two prefill kernels.
 constexpr int kDenseRows = 256;
 constexpr int kSparseRows = 64;
+// The short form of the dense kernel (head_dim 64): query rows per workgroup,
+// LDS stages, keys per tile, workgroups resident per CU.
+constexpr int kShortRows = 128;
+constexpr int kShortStages = 5;
+constexpr int kShortTileKeys = 32;
+constexpr int kShortPerCu = 3;
 // LDS stages of the two prefill kernels: KV tiles resident per workgroup
 // (dense), K tiles and V tiles resident per workgroup (block-sparse: the K
 // ring runs one tile ahead of the V ring).

@@ -303,9 +303,9 @@ struct TileDma {
     if (k0 + TN <= s.len) {
       // whole tile inside the sequence
       const uint32_t k0u = (uint32_t)__builtin_amdgcn_readfirstlane(k0);
-      // (scalar base + lane offset pays in the dense kernel; the block-sparse one,
+      // (scalar base + lane offset pays in the dense kernels; the block-sparse one,
       // whose base changes with every listed block, measured faster with the sum in vector registers)
-      constexpr bool kScalarBase = NW >= 8;
+      constexpr bool kScalarBase = NW >= 4;
       const uint64_t kt_u = s.k_base + (uint64_t)k0u * k_pitch, vt_u = s.v_base + (uint64_t)k0u * v_pitch;
       const uint64_t kt_s = kScalarBase ? uniform64(kt_u) : 0, vt_s = kScalarBase ? uniform64(vt_u) : 0;
 #pragma unroll
@@ -1157,6 +1157,395 @@ dense_kernel(const PrefillParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Dense, short form (head_dim 64): workgroups of 4 wavefronts (128 query rows
+// per item), three to a CU, KV tiles of 32 keys in a ring of five stages
+// (40 KiB of LDS per workgroup at head_dim 64).
+//
+// dense_kernel keeps one 8-wave workgroup per CU, two wavefronts per SIMD.  At
+// head_dim 64 the softmax arithmetic outweighs the matrix work (56 vector
+// instructions against 8 MFMAs per 32 x 32 block of scores) and a wave's
+// registers (O, S, Q^T, P: 163 in all) leave room for a third wavefront per
+// SIMD, which fills issue slots that two leave empty; three independent
+// workgroups also run one another's item boundaries under their tile loops.
+// Measured against dense_kernel at head_dim 64 (HIP events, same box): 3 to 8 %
+// faster on launches of eight rounds or more (4 x 8192 tokens, 32 heads: 1158
+// against 1190 us), 6 to 11 % on 16 sequences of 2048 / 512 tokens, 4 to 10 % on
+// launches of at most one workgroup per CU; slower where the item count is a
+// round and a bit (1024 or 2048 items on 768 slots), which the launcher leaves
+// to dense_kernel.  At head_dim 96 and 128 a wave needs 185 / 218 registers, two
+// fit a SIMD either way, and this form measured equal or slower: it is built
+// for head_dim 64 only.  The price is twice the tile traffic from the L2s per
+// query row.
+//
+// The same half-tile software pipeline as dense_kernel, a tile now being one
+// half: at position h a wave forms S(h+1) = K(h+1) Q^T together with the second
+// half of the exponentials of S(h), then O += V(h)^T P(h)^T together with the
+// first half of those of S(h+1), and reads the first K fragments of tile h+2
+// along the way.  Tile j is requested at the top of position j - 4 into stage
+// j % 5, the stage of tile j - 5, which every wave has left by then (barrier);
+// at the top of position h tiles up to h+2 must have landed, tile h+3 may still
+// be in flight (counted wait, loads retire in issue order).  Score registers
+// alternate with the position's parity and the ring has five stages, so the
+// tile loop is unrolled ten times.
+template <typename T, int D>
+__global__ void __launch_bounds__(kShortRows * 2) __attribute__((amdgpu_waves_per_eu(kShortPerCu)))
+dense_short_kernel(const PrefillParams p) {
+  constexpr int NW = kShortRows / 32, NS = kShortStages, TN = kShortTileKeys;
+  static_assert(NW == 4 && NS == 5 && TN == 32, "stage use at the item boundary assumes this shape");
+  using G = RowGeom<D>;
+  using F = SwizzledFrags<D>;
+  using DMA = TileDma<T, D, NW, NS, TN>;
+  constexpr int BM = 32 * NW;
+  constexpr int TILEB = DMA::TILEB, VBASE = DMA::VBASE, IPW = DMA::IPW;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  F fr;
+  fr.init(lane, (uint32_t)(uintptr_t)smem, VBASE);
+  DMA dma;
+  dma.init(p, lane, wave);
+  const int causal = p.causal;
+  const float scale = p.scale;
+
+  struct Item {
+    int len, q0, n_tiles;
+    const T* qp;
+    T* op;
+    float* lp;
+    KvSrc<T> kv;
+  };
+  const int grid = gridDim.x;
+  int round = 0, base = 0;
+  auto next_item = [&](Item& it) __attribute__((always_inline)) -> bool {
+    while (base < p.n_items) {
+      int w = blockIdx.x;
+      if ((round & 1) && (grid & 7) == 0) w = (((grid >> 3) - 1 - (w >> 3)) << 3) | (w & 7);
+      const int bid = base + w;
+      base += grid;
+      ++round;
+      ItemGeo g;
+      if (bid < p.n_items && item_geo<BM>(p, bid, g)) {
+        it.len = g.len;
+        it.q0 = g.qt * BM;
+        it.n_tiles = (g.len + TN - 1) / TN;
+        if (causal) it.n_tiles = min(it.n_tiles, (it.q0 + BM + TN - 1) / TN);
+        it.qp = reinterpret_cast<const T*>(p.q) + g.q_off + g.h * p.q_sh;
+        it.op = reinterpret_cast<T*>(p.o) + g.o_off + g.h * p.o_sh;
+        it.lp = p.lse ? p.lse + g.lse_off + g.h * p.lse_sh : nullptr;
+        it.kv = DMA::source(reinterpret_cast<const T*>(p.k) + g.k_off + g.kvh * p.k_sh,
+                            reinterpret_cast<const T*>(p.v) + g.v_off + g.kvh * p.v_sh, g.len);
+        return true;
+      }
+    }
+    return false;
+  };
+  // Q^T operands of an item and its first tile; tiles 1 to 3 follow from
+  // request_tile<1..3>.  Nothing waits here (loads from inline assembly, see dense_kernel).
+  auto request_item = [&](const Item& it, i32x4 (&Q)[G::KSTEPS]) __attribute__((always_inline)) {
+    const int row = min(it.q0 + 32 * wave + fr.lq, it.len - 1);
+    const T* qr = it.qp + (int64_t)row * p.q_ss + 8 * fr.lh;
+#pragma unroll
+    for (int c = 0; c < G::KSTEPS; ++c)
+      asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(Q[c]) : "v"(qr), "n"(32 * c));
+    if (0 < it.n_tiles) dma.template tile<0>(it.kv, 0);
+  };
+  auto request_tile = [&](auto j_c, const Item& it) __attribute__((always_inline)) {
+    constexpr int J = decltype(j_c)::value;
+    if (J < it.n_tiles) dma.template tile<J>(it.kv, J * TN);
+  };
+
+  Item cur;
+  i32x4 Qf[G::KSTEPS];
+  f32x16 O[G::NDB];
+  float m, l, m_neg;
+  int len, n_tiles, q0w, qrow, row_lim, H_w;
+  int tail_h;  // first position (> 0) at whose top no further tile is requested
+  f32x16 S[2];
+  constexpr int KR = G::KSTEPS < 4 ? G::KSTEPS : 4;
+  i32x4 kf[KR];
+
+  auto mask_half = [&](int hh, f32x16& Sx) __attribute__((always_inline)) {
+    const int k0h = hh * 32;
+    if ((k0h + 32 > len) || (causal && k0h + 31 > q0w)) {
+      const int t = row_lim - k0h - 8 * fr.lh;
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (16 * (r >> 3) + (r & 7) > t) Sx[r] = -INFINITY;
+    }
+  };
+
+  constexpr float kRowSumLimit = 4096.f;
+  uint32_t Pb[2][8];
+  float rsv[2];
+  float e_p0, e_u1;
+  auto exp_first = [&](const f32x16& Sx, int i, float mn) __attribute__((always_inline)) {
+    e_p0 = fast_exp2(fmaf(Sx[2 * i], scale, mn));
+    e_u1 = fmaf(Sx[2 * i + 1], scale, mn);
+  };
+  auto exp_second = [&](int i, uint32_t (&Pd)[8], float& rs) __attribute__((always_inline)) {
+    const float p1 = fast_exp2(e_u1);
+    rs = i == 0 ? e_p0 + p1 : rs + (e_p0 + p1);
+    Pd[i] = Elem<T>::pack2(e_p0, p1);
+  };
+  float su0[2], su1[2], sp0[2], sp1[2], st;
+  auto soft_slice = [&](int c, const f32x16& Sx, int i0, uint32_t (&Pd)[8], float& rs, float mn) __attribute__((always_inline)) {
+    const int j = (c + 1) / 2;
+    if (c == 0) {
+      su0[0] = fmaf(Sx[2 * i0], scale, mn);
+      su1[0] = fmaf(Sx[2 * i0 + 1], scale, mn);
+      sp0[0] = fast_exp2(su0[0]);
+      return;
+    }
+    if (c & 1) {
+      const int k = (c - 1) / 2, sl = k & 1;
+      sp1[sl] = fast_exp2(su1[sl]);
+      if (k > 0) rs = (i0 == 0 && k == 1) ? st : rs + st;
+      if (k < 3) {
+        su0[sl ^ 1] = fmaf(Sx[2 * (i0 + k + 1)], scale, mn);
+        su1[sl ^ 1] = fmaf(Sx[2 * (i0 + k + 1) + 1], scale, mn);
+      } else {
+        const float t2 = sp0[sl] + sp1[sl];
+        Pd[i0 + 3] = Elem<T>::pack2(sp0[sl], sp1[sl]);
+        rs += t2;
+      }
+    } else {
+      const int sl = j & 1;
+      sp0[sl] = fast_exp2(su0[sl]);
+      st = sp0[sl ^ 1] + sp1[sl ^ 1];
+      Pd[i0 + j - 1] = Elem<T>::pack2(sp0[sl ^ 1], sp1[sl ^ 1]);
+    }
+  };
+  auto exact_fix = [&](const f32x16& Sx, uint32_t (&Pd)[8], float& rs) __attribute__((always_inline)) {
+    float mx = Sx[0];
+#pragma unroll
+    for (int r = 1; r < 16; ++r) mx = fmaxf(mx, Sx[r]);
+    mx = max_with_other_half(mx);
+    const float m_new = fmaxf(m, mx * scale);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = fast_exp2(m - m_safe);
+    l *= alpha;
+#pragma unroll
+    for (int db = 0; db < G::NDB; ++db) O[db] *= alpha;
+    m = m_new;
+    m_neg = -m_safe;
+    rs = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float p0 = fast_exp2(fmaf(Sx[2 * i], scale, -m_safe));
+      const float p1 = fast_exp2(fmaf(Sx[2 * i + 1], scale, -m_safe));
+      rs += p0 + p1;
+      Pd[i] = Elem<T>::pack2(p0, p1);
+    }
+  };
+
+  // position h; J = h % 10: stage J % 5, score registers S[J & 1]
+  auto half_step = [&](auto j_c, int h) __attribute__((always_inline)) {
+    constexpr int J = decltype(j_c)::value;
+    if (h >= H_w) return;
+    constexpr int TS = J % NS, KB = J & 1;
+    constexpr uint32_t KOFF = ((TS + 1) % NS) * TILEB, VOFF = TS * TILEB, K2OFF = ((TS + 2) % NS) * TILEB;
+    f32x16& Sc = S[KB];
+    f32x16& Sn = S[KB ^ 1];
+    uint32_t (&Pc)[8] = Pb[KB];
+    uint32_t (&Pn)[8] = Pb[KB ^ 1];
+    __builtin_amdgcn_s_setprio(3);
+    i32x4 vf[G::NDB];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      if (c < G::KSTEPS) {
+        const f32x16 acc = (c == 0) ? (f32x16){0} : Sn;
+        Sn = Elem<T>::mfma(kf[c % KR], Qf[c], acc);
+        if (c + KR < G::KSTEPS) kf[c % KR] = fr.load_k(KOFF, 0, c + KR);
+      }
+      if (c >= 8 - G::NDB) vf[c - (8 - G::NDB)] = fr.load_v(VOFF, 0, c - (8 - G::NDB));
+      soft_slice(c, Sc, 4, Pc, rsv[KB], m_neg);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("" : "+v"(Pc[4]), "+v"(Pc[5]), "+v"(Pc[6]), "+v"(Pc[7]), "+v"(rsv[KB]));
+    if (__builtin_amdgcn_ballot_w64(!(rsv[KB] <= kRowSumLimit)) != 0) exact_fix(Sc, Pc, rsv[KB]);
+    l += rsv[KB];
+    mask_half(h + 1, Sn);
+    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int sl = 0; sl < 8; ++sl) {
+      if (sl < 2 * G::NDB) {
+        const int kk = sl / G::NDB, db = sl % G::NDB;
+        const i32x4 pf = {(int)Pc[4 * kk], (int)Pc[4 * kk + 1], (int)Pc[4 * kk + 2], (int)Pc[4 * kk + 3]};
+        O[db] = Elem<T>::mfma(vf[db], pf, O[db]);
+        if (kk == 0) vf[db] = fr.load_v(VOFF, 1, db);
+      }
+      if (sl >= 4 && sl - 4 < KR) kf[sl - 4] = fr.load_k(K2OFF, 0, sl - 4);
+      // (for the last position of a wave Sn holds scores of stale LDS contents: the results are never used)
+      soft_slice(sl, Sn, 0, Pn, rsv[KB ^ 1], m_neg);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("" : "+v"(Pn[0]), "+v"(Pn[1]), "+v"(Pn[2]), "+v"(Pn[3]), "+v"(rsv[KB ^ 1]));
+  };
+
+  // top of position h (> 0), then the position
+  auto pos = [&](auto j_c, int h) __attribute__((always_inline)) {
+    constexpr int J = decltype(j_c)::value;
+    if (h + NS - 1 < n_tiles) {
+      // tiles up to h+2 landed (requested at least two positions ago); tile h+3 may still fly
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 4) * 2 * IPW));
+      __syncthreads();
+      dma.template tile<(J + NS - 1) % NS>(cur.kv, (h + NS - 1) * TN);
+    } else if (h == tail_h) {
+      // nothing left to request: one full wait and one barrier publish what is
+      // still on its way, and the waves run to the end of the item on their own
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+      __syncthreads();
+    }
+    half_step(j_c, h);
+  };
+
+  // ---- normalise, transpose through LDS, coalesced 16-byte stores (as in
+  // dense_kernel; the staging area is the last stage: waves 0, 1 in its K tile,
+  // waves 2, 3 in its V tile)
+  constexpr int DBP = (G::NDB + 1) / 2;
+  constexpr int SROW = DBP * 64;
+  constexpr int CH = SROW / 16;
+  auto write_out = [&](auto&& after_pass0, auto&& after_pass1) __attribute__((always_inline)) {
+    static_assert(2 * 32 * SROW <= TILEB, "two waves stage inside one tile");
+    auto sswz = [](int row) { return SROW == 128 ? ((row >> 1) & 7) : ((row >> 2) & 3); };
+    int lane_o = lane, lq_o = fr.lq, lh_o = fr.lh;
+    asm volatile("" : "+v"(lane_o), "+v"(lq_o), "+v"(lh_o));
+    const float l_tot = sum_with_other_half(l);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (cur.lp && lh_o == 0 && qrow < len)
+      cur.lp[(int64_t)qrow * p.lse_ss] = l_tot > 0.f ? m + fast_log2(l_tot) : -INFINITY;
+    unsigned char* stage = smem + (wave < 2 ? 0 : VBASE) + (NS - 1) * TILEB + (wave & 1) * 32 * SROW;
+#pragma unroll
+    for (int ps = 0; ps < 2; ++ps) {
+#pragma unroll
+      for (int dl = 0; dl < DBP; ++dl) {
+        const int db = ps * DBP + dl;
+        if (db < G::NDB) {
+#pragma unroll
+          for (int gq = 0; gq < 4; ++gq) {
+            const int c = 4 * dl + gq;
+            i32x2 w;
+            w[0] = (int)Elem<T>::pack2(O[db][4 * gq] * inv, O[db][4 * gq + 1] * inv);
+            w[1] = (int)Elem<T>::pack2(O[db][4 * gq + 2] * inv, O[db][4 * gq + 3] * inv);
+            *reinterpret_cast<i32x2*>(stage + lq_o * SROW + ((c ^ sswz(lq_o)) << 4) + 8 * lh_o) = w;
+          }
+        }
+      }
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int i = 0; i < 32 * CH / 64; ++i) {
+        const int idx = lane_o + 64 * i;
+        const int row = idx / CH, ch = idx % CH;
+        const int och = ps * CH + ch;
+        if (och < G::NCH && q0w + row < len) {
+          const i32x4 val = *reinterpret_cast<const i32x4*>(stage + row * SROW + ((ch ^ sswz(row)) << 4));
+          T* dst = cur.op + (int64_t)(q0w + row) * p.o_ss + och * 8;
+          // (from assembly, so that no counted wait of the compiler's sits between these stores and the tile requests around them)
+          asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1" : : "v"(dst), "v"(val) : "memory");
+        }
+      }
+      asm volatile("" ::: "memory");
+      if (ps == 0)
+        after_pass0();
+      else
+        after_pass1();
+    }
+  };
+
+  bool have = next_item(cur);
+  if (have) {
+    request_item(cur, Qf);
+    request_tile(ic<1>{}, cur);
+    request_tile(ic<2>{}, cur);
+    request_tile(ic<3>{}, cur);
+  }
+  while (have) {
+    len = cur.len;
+    n_tiles = cur.n_tiles;
+    q0w = cur.q0 + 32 * wave;
+    qrow = q0w + fr.lq;
+    row_lim = causal ? min(qrow, len - 1) : len - 1;
+    H_w = (len + 31) / 32;
+    if (causal) H_w = min(H_w, q0w / 32 + 1);
+    H_w = min(H_w, n_tiles);
+    if (q0w >= len) H_w = 0;
+    tail_h = max(1, n_tiles - (NS - 1));
+#pragma unroll
+    for (int db = 0; db < G::NDB; ++db) O[db] = (f32x16){0};
+    m = -INFINITY;
+    m_neg = 0.f;
+    l = 0.f;
+
+    // Q and tiles 0 to 2 must have landed (position 0 reads K of tiles 1 and
+    // 2).  They were requested in the order Q, tile 0, [stores], tile 1,
+    // [stores], tile 2, tile 3, and everything retires in that order: when tile
+    // 3 exists its loads are the youngest and may stay in flight.
+    if (NS - 2 < n_tiles)
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * IPW));
+    else
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+#pragma unroll
+    for (int c = 0; c < G::KSTEPS; ++c) asm volatile("" : "+v"(Qf[c]));
+    __syncthreads();
+    if (NS - 1 < n_tiles) dma.template tile<NS - 1>(cur.kv, (NS - 1) * TN);
+    if (H_w > 0) {
+      f32x16 acc = (f32x16){0};
+#pragma unroll
+      for (int c = 0; c < G::KSTEPS; ++c) acc = Elem<T>::mfma(fr.load_k(0u, 0, c), Qf[c], acc);
+      S[0] = acc;
+      mask_half(0, S[0]);
+      exact_fix(S[0], Pb[0], rsv[0]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        exp_first(S[0], i, m_neg);
+        exp_second(i, Pb[0], rsv[0]);
+      }
+#pragma unroll
+      for (int c = 0; c < KR; ++c) kf[c] = fr.load_k(1u * TILEB, 0, c);
+    }
+
+    half_step(ic<0>{}, 0);
+    for (int h = 1; h < n_tiles; h += 10) {
+      pos(ic<1>{}, h);
+      if (h + 1 >= n_tiles) break;
+      pos(ic<2>{}, h + 1);
+      if (h + 2 >= n_tiles) break;
+      pos(ic<3>{}, h + 2);
+      if (h + 3 >= n_tiles) break;
+      pos(ic<4>{}, h + 3);
+      if (h + 4 >= n_tiles) break;
+      pos(ic<5>{}, h + 4);
+      if (h + 5 >= n_tiles) break;
+      pos(ic<6>{}, h + 5);
+      if (h + 6 >= n_tiles) break;
+      pos(ic<7>{}, h + 6);
+      if (h + 7 >= n_tiles) break;
+      pos(ic<8>{}, h + 7);
+      if (h + 8 >= n_tiles) break;
+      pos(ic<9>{}, h + 8);
+      if (h + 9 >= n_tiles) break;
+      pos(ic<0>{}, h + 9);
+    }
+    __builtin_amdgcn_s_setprio(0);
+    __syncthreads();  // every wave is done with the tiles
+
+    Item nxt = cur;
+    const bool more = next_item(nxt);
+    if (more) request_item(nxt, Qf);
+    write_out([&]() __attribute__((always_inline)) { if (more) request_tile(ic<1>{}, nxt); },
+              [&]() __attribute__((always_inline)) {
+                if (more) {
+                  request_tile(ic<2>{}, nxt);
+                  request_tile(ic<3>{}, nxt);
+                }
+              });
+    cur = nxt;
+    have = more;
+  }
+}
+
 template <int D, int NW, int NS, int TN>
 constexpr size_t prefill_lds_bytes() {
   const size_t pipe = (size_t)NS * 2 * TN * SwizzledFrags<D>::ROWB;
@@ -1164,8 +1553,39 @@ constexpr size_t prefill_lds_bytes() {
   return pipe > epi ? pipe : epi;
 }
 
+// Does the short form pay for this launch (head_dim 64)?  n = its 128-row work
+// items.  Yes when every workgroup has a CU to itself (twice as many CUs busy
+// as with 256-row items), and when the launch is eight rounds of three
+// workgroups per CU or more; in between, the last, partly filled round of the
+// short form costs more than its third wavefront per SIMD gains (measured on 1
+// to 32 sequences of 256 to 8192 tokens, causal and not).
+inline bool short_form_pays(long long n, int cus) {
+  return cus > 0 && (n <= cus || n >= 8LL * kShortPerCu * cus);
+}
+
+template <typename T, int D>
+int launch_short(const PrefillParams& p, long long items, int cus, hipStream_t s) {
+  auto kern = dense_short_kernel<T, D>;
+  constexpr size_t lds = prefill_lds_bytes<D, kShortRows / 32, kShortStages, kShortTileKeys>();
+  static_assert(kShortPerCu * lds <= 160 * 1024, "kShortPerCu workgroups share a CU's LDS");
+  static LdsLimitOnce lds_once;
+  if (const int e = raise_lds_limit(lds_once, reinterpret_cast<const void*>(kern), (int)lds)) return e;
+  PrefillParams pp = p;
+  pp.n_qtiles = (p.max_seqlen + kShortRows - 1) / kShortRows;
+  pp.n_items = (int)items;
+  long long grid = items;
+  if (grid > (long long)kShortPerCu * cus) grid = (long long)kShortPerCu * cus;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kShortRows * 2), lds, s, pp);
+  return (int)hipGetLastError();
+}
+
 template <typename T, int D, bool SPARSE>
 int launch_one(const PrefillParams& p, hipStream_t s) {
+  if constexpr (!SPARSE && D == 64) {
+    const int cus = device_cu_count();
+    const long long n = (long long)((p.max_seqlen + kShortRows - 1) / kShortRows) * p.hq * p.batch;
+    if (short_form_pays(n, cus)) return launch_short<T, D>(p, n, cus, s);
+  }
   constexpr int NW = (SPARSE ? kSparseRows : kDenseRows) / 32;
   constexpr int NS = SPARSE ? kSparseStages : kDenseStages;
   constexpr int TN = SPARSE ? kSparseTileKeys : kTileN;
