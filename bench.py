@@ -141,12 +141,21 @@ def _fwd_args(q, k, v, o, lse, causal):
 
 # (batch, heads, sequence length) of the dense causal workload; --dense-shape replaces it for profiling other
 # shapes (the headline line of the default run is always the benchmark's own configuration)
-DENSE_SHAPE = (4, 32, 8192)
+DENSE_SHAPE = (4, 32, 8192, 128)
+
+
+def _dense_kernel_name(D):
+    if D == 128:
+        return KERNELS["dense_causal"]
+    name = _NS + "12dense_kernelIDF16bLi%dEEEvNS_13PrefillParamsE" % D
+    if D == 64:   # the launcher picks the form from the number of work items
+        name += " or " + KERNELS["c1_dense_noncausal_small"]
+    return name
 
 
 def run_dense_causal(steps, warmup):
     import tritonops_amd as ta
-    (B, H, S), D = DENSE_SHAPE, 128
+    B, H, S, D = DENSE_SHAPE
     q, k, v = (_randn((B, H, S, D), s) for s in (0, 1, 2))
     fn = lambda: ta.flash_attention(q, k, v, causal=True, return_lse=True)
     ms = _time_steps(fn, steps, warmup)
@@ -169,8 +178,8 @@ def run_dense_causal(steps, warmup):
         "max_abs_err": err, "max_abs_err_lse2": err_lse,
         "err_sample": "o and lse of 3 (batch, head) units x 4 blocks of 64 query rows against fp32 torch math on the device",
         "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "kernel": KERNELS["dense_causal"]},
-        "config": {"workload": "dense causal flash-attention fwd bf16 B=%d H=%d S=%d D=128, o bf16 + lse fp32" % (B, H, S),
+                     "unit": "TFLOP/s", "kernel": _dense_kernel_name(D)},
+        "config": {"workload": "dense causal flash-attention fwd bf16 B=%d H=%d S=%d D=%d, o bf16 + lse fp32" % (B, H, S, D),
                    "flop_per_step": flop, "flop_reference_convention_4BHS2D": 4.0 * B * H * S * S * D},
     }
 
@@ -197,7 +206,7 @@ def run_c1_small(steps, warmup):
         "err_sample": "all of o against fp32 softmax(q k^T / 8) v on the fp32 inputs (the kernel sees their bf16 cast)",
         "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "kernel": KERNELS["c1_dense_noncausal_small"]},
-        "config": {"workload": "dense non-causal attention fwd B=1 H=4 S=256 D=64 (the reference's CPU case; 4 work items, "
+        "config": {"workload": "dense non-causal attention fwd B=1 H=4 S=256 D=64 (the reference's CPU case; 8 work items, "
                                "launch-latency bound on a GPU), bf16 cast of fp32 N(0,1) inputs from seed 0",
                    "flop_per_step": flop},
     }
@@ -987,15 +996,19 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also launch one elementwise copy of 1 GiB (2 GiB of HBM traffic) as the reference "
                          "dispatch for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
-    ap.add_argument("--dense-shape", default=None, metavar="B,H,S",
-                    help="batch, heads and sequence length of the dense_causal workload instead of the benchmark's "
-                         "4,32,8192 (S a multiple of 64, at least 256; for profiling other shapes)")
+    ap.add_argument("--dense-shape", default=None, metavar="B,H,S[,D]",
+                    help="batch, heads, sequence length and head_dim of the dense_causal workload instead of the "
+                         "benchmark's 4,32,8192,128 (S a multiple of 64, at least 256; D 64, 96 or 128; for "
+                         "profiling other shapes)")
     a = ap.parse_args()
     if a.dense_shape:
         global DENSE_SHAPE
-        DENSE_SHAPE = tuple(int(x) for x in a.dense_shape.split(","))
-        if len(DENSE_SHAPE) != 3 or min(DENSE_SHAPE) < 1 or DENSE_SHAPE[2] % 64 or DENSE_SHAPE[2] < 256:
-            sys.exit("bench.py: --dense-shape takes B,H,S with S a multiple of 64, at least 256")
+        sh = tuple(int(x) for x in a.dense_shape.split(","))
+        if len(sh) == 3:
+            sh += (128,)
+        if len(sh) != 4 or min(sh) < 1 or sh[2] % 64 or sh[2] < 256 or sh[3] not in (64, 96, 128):
+            sys.exit("bench.py: --dense-shape takes B,H,S[,D] with S a multiple of 64, at least 256, and D 64, 96 or 128")
+        DENSE_SHAPE = sh
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the attention path shards over batch and "
                  "heads without communication); run with --gpus 1")
@@ -1025,7 +1038,7 @@ def main():
         t = traffic.get(r["name"], {})
         fresh = t.get("kernel") == rf["kernel"]
         rf["traffic"] = t.get("hbm_bytes_per_launch") if fresh else None
-        rf["traffic_source"] = ("profiles/hbm_traffic.json, measured at commit %s" % traffic.get("_commit", "?")
+        rf["traffic_source"] = ("profiles/hbm_traffic.json, measured at commit %s" % t.get("commit", traffic.get("_commit", "?"))
                                 if fresh else "no counter run of this kernel on file")
         r["parity_ok"], r["parity_bars"] = _parity(r)
         results.append(r)
