@@ -1,9 +1,9 @@
-"""The two forms of the dense forward at head_dim 64: launches of at most one
-128-row work item per CU and launches of eight rounds or more run the short
-form (4-wave workgroups, three to a CU); everything in between runs the
-8-wave kernel that also serves head_dim 96 and 128.  Both against the oracle,
-and against each other bit for bit: a row's keys are met in the same order,
-32 at a time, in either form."""
+"""The two forms of the dense forward at head_dim 64: the short form (4-wave
+workgroups of 128 rows, three to a CU) and the 8-wave kernel that also serves
+head_dim 96 and 128; the launcher picks one per launch from the number of work
+items (prefill.hip, short_form_pays).  Both against the oracle, and against
+each other bit for bit: a row's keys are met in the same order, 32 at a time,
+in either form."""
 import pytest
 import torch
 
@@ -12,12 +12,6 @@ from tests.util import LSE_TOL, TOL, assert_close, cu_from, randn
 
 pytestmark = pytest.mark.gpu
 
-SHORT_ROWS, SHORT_PER_CU, ROUNDS = 128, 3, 8
-
-
-def _items(batch, heads, max_len):
-    return batch * heads * ((max_len + SHORT_ROWS - 1) // SHORT_ROWS)
-
 
 def _cus():
     from tritonops_amd import _lib
@@ -25,21 +19,44 @@ def _cus():
 
 
 def _runs_short_form(batch, heads, max_len):
-    n, cus = _items(batch, heads, max_len), _cus()
-    return n <= cus or n >= ROUNDS * SHORT_PER_CU * cus
+    """The launcher's choice, restated (prefill.hip: short_form_cost / short_form_pays)."""
+    cus = _cus()
+    n128 = batch * heads * ((max_len + 127) // 128)
+    n256 = batch * heads * ((max_len + 255) // 256)
+    if n128 <= cus:
+        return True
+    grid = 3 * cus
+    q, r = divmod(n128, grid)
+    rate = {1: 0.4, 2: 0.7, 3: 1.0}
+    worst = 0.0
+    for c in (0, cus - 1):
+        items = [q + (1 if c + k * cus < r else 0) for k in range(3)]
+        t, done = 0.0, 0
+        for live in (3, 2, 1):
+            upto = items[live - 1]
+            if upto > done:
+                t += (upto - done) * live / rate[live]
+                done = upto
+        worst = max(worst, t)
+    return worst < 2.3 * ((n256 + cus - 1) // cus)
 
 
-LENS = [0, 1, 300, 257, 2049, 511, 0, 1500, 31, 1024, 513, 2500, 255, 256, 1000, 2047, 64, 700, 1, 1280, 129, 127, 128,
-        33, 2304, 96]
+LENS_LONG = [0, 1, 300, 257, 2049, 511, 0, 1500, 31, 1024, 513, 2500, 255, 256, 1000, 2047, 64, 700, 1, 1280, 129, 127,
+             128, 33, 2304, 96]
+LENS_SHORT = [512, 0, 1, 300, 257, 511, 31, 500, 255, 256, 64, 129, 127, 128, 33, 96, 385, 383, 200, 77, 5, 450, 321, 100,
+              160, 192, 224, 288, 352, 416, 480, 17]
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("heads_q,short_form", [(16, True), (4, False)])
-def test_ragged_packed_batch_in_either_form(heads_q, short_form, dtype):
+@pytest.mark.parametrize("lens,heads_q,short_form", [(LENS_LONG, 16, True), (LENS_SHORT, 8, False)])
+def test_ragged_packed_batch_in_either_form(lens, heads_q, short_form, dtype):
+    """26 sequences of up to 2500 tokens x 16 heads (8320 work items of 128 rows: ten full rounds and most of an
+    eleventh); 32 sequences of up to 512 tokens x 8 heads (1024 items of 128 rows are one round and a third, 512 items of
+    256 rows two even rounds: the 8-wave kernel)."""
     import tritonops_amd as ta
 
-    lens = torch.tensor(LENS, dtype=torch.int32)
-    assert _runs_short_form(len(LENS), heads_q, int(lens.max())) == short_form, "sizes no longer select the intended form"
+    lens = torch.tensor(lens, dtype=torch.int32)
+    assert _runs_short_form(len(lens), heads_q, int(lens.max())) == short_form, "sizes no longer select the intended form"
     cu = cu_from(lens)
     T = int(cu[-1])
     q, k, v = randn((1, T, heads_q, 64), 4, dtype), randn((1, T, 2, 64), 5, dtype), randn((1, T, 2, 64), 6, dtype)
@@ -56,8 +73,9 @@ def test_ragged_packed_batch_in_either_form(heads_q, short_form, dtype):
 
 @pytest.mark.parametrize("causal", [True, False])
 def test_the_two_forms_agree_bit_for_bit(causal):
-    """48 sequences of 512 tokens (6144 work items: short form) and the first 8
-    of them on their own (1024 items: the 8-wave kernel)."""
+    """48 sequences of 512 tokens (6144 work items of 128 rows, eight even rounds: short form) and the first 8
+    of them on their own (1024 items, a round and a third, against two even rounds of 256-row items: the 8-wave
+    kernel)."""
     import tritonops_amd as ta
 
     B, H, S, D = 48, 32, 512, 64

@@ -1172,8 +1172,8 @@ dense_kernel(const PrefillParams p) {
 // faster on launches of eight rounds or more (4 x 8192 tokens, 32 heads: 1158
 // against 1190 us), 6 to 11 % on 16 sequences of 2048 / 512 tokens, 4 to 10 % on
 // launches of at most one workgroup per CU; slower where the item count is a
-// round and a bit (1024 or 2048 items on 768 slots), which the launcher leaves
-// to dense_kernel.  At head_dim 96 and 128 a wave needs 185 / 218 registers, two
+// round and a bit (1024 items on 768 slots) while dense_kernel's rounds come
+// out even, which the launcher works out per launch (short_form_pays).  At head_dim 96 and 128 a wave needs 185 / 218 registers, two
 // fit a SIMD either way, and this form measured equal or slower: it is built
 // for head_dim 64 only.  The price is twice the tile traffic from the L2s per
 // query row.
@@ -1553,14 +1553,45 @@ constexpr size_t prefill_lds_bytes() {
   return pipe > epi ? pipe : epi;
 }
 
-// Does the short form pay for this launch (head_dim 64)?  n = its 128-row work
-// items.  Yes when every workgroup has a CU to itself (twice as many CUs busy
-// as with 256-row items), and when the launch is eight rounds of three
-// workgroups per CU or more; in between, the last, partly filled round of the
-// short form costs more than its third wavefront per SIMD gains (measured on 1
-// to 32 sequences of 256 to 8192 tokens, causal and not).
-inline bool short_form_pays(long long n, int cus) {
-  return cus > 0 && (n <= cus || n >= 8LL * kShortPerCu * cus);
+// Which form for a head_dim-64 launch?  A model of how long the busiest CU
+// works, in units of one 128-row item at full occupancy.  Short form: the grid
+// is kShortPerCu workgroups per CU, workgroup w sits on CU w % cus and walks
+// items w, w + grid, ...; the first n % grid workgroups have one item more than
+// the others.  Three resident workgroups keep a CU busy; when the ones with
+// fewer items have finished, two run at 0.7 and a lone one at 0.4 of that rate.
+// Long form: one 256-row item after another per CU, each worth 2.3 items of the
+// short form (twice the rows at about 13 % less per row).  The three constants
+// are fitted to HIP-event timings of both forms on 1 to 48 sequences of 256 to
+// 8192 tokens with 12, 20 and 32 heads, causal and not: against the faster
+// form of each launch the choice costs 0.7 % in the geometric mean (always the
+// long form: 8.5 %, always the short form: 2.5 %).
+inline double short_form_cost(long long n, int cus) {
+  const long long grid = (long long)kShortPerCu * cus;
+  const long long q = n / grid, r = n % grid;
+  static_assert(kShortPerCu == 3, "the rates below are those of one, two and three workgroups");
+  const double rate[kShortPerCu + 1] = {0.0, 0.4, 0.7, 1.0};
+  double worst = 0.0;
+  for (const int c : {0, cus - 1}) {   // items per workgroup fall with the workgroup id: the ends of the range suffice
+    long long items[kShortPerCu];
+    for (int k = 0; k < kShortPerCu; ++k) items[k] = q + ((long long)c + (long long)k * cus < r ? 1 : 0);
+    // (items[0] >= items[1] >= items[2]) phases: all three until the shortest is done, then two, then one
+    double t = 0.0;
+    long long done = 0;
+    for (int live = kShortPerCu; live >= 1; --live) {
+      const long long upto = items[live - 1];
+      if (upto > done) {
+        t += (double)(upto - done) * live / rate[live];
+        done = upto;
+      }
+    }
+    worst = t > worst ? t : worst;
+  }
+  return worst;
+}
+inline bool short_form_pays(long long n128, long long n256, int cus) {
+  if (cus <= 0) return false;
+  if (n128 <= cus) return true;   // a CU per workgroup: twice as many CUs busy as with 256-row items
+  return short_form_cost(n128, cus) < 2.3 * (double)((n256 + cus - 1) / cus);
 }
 
 template <typename T, int D>
@@ -1584,7 +1615,7 @@ int launch_one(const PrefillParams& p, hipStream_t s) {
   if constexpr (!SPARSE && D == 64) {
     const int cus = device_cu_count();
     const long long n = (long long)((p.max_seqlen + kShortRows - 1) / kShortRows) * p.hq * p.batch;
-    if (short_form_pays(n, cus)) return launch_short<T, D>(p, n, cus, s);
+    if (short_form_pays(n, (long long)p.n_qtiles * p.hq * p.batch, cus)) return launch_short<T, D>(p, n, cus, s);
   }
   constexpr int NW = (SPARSE ? kSparseRows : kDenseRows) / 32;
   constexpr int NS = SPARSE ? kSparseStages : kDenseStages;
