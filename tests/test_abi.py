@@ -266,6 +266,10 @@ def test_split_heuristic(lib):
         assert t % 64 == 0 and 64 <= t <= 2048
     assert f(64, 8, 32768, 256) == 2048          # plenty of work: the longest chunk
     assert f(1, 8, 32768, 256) == 512            # little work: the shortest chunk worth a partial result
+    assert f(1, 8, 8192, 256) == 256             # ... which is shorter where a sequence still makes at most 32 chunks
+    assert f(4, 8, 8192, 256) == 256
+    assert f(8, 8, 8192, 256) == 512
+    assert f(1, 8, 12288, 256) == 384
     assert f(4, 8, 32768, 256) == 1024           # in between: about half a resident round's share
     assert f(1, 1, 1 << 20, 256) == 1024
 

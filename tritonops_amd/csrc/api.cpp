@@ -548,14 +548,19 @@ int mi_decode_choose_split_tokens(int batch, int heads_kv, int max_seqlen, int n
   // The dense kernel deals the live chunks to one resident round of wavefronts
   // (8 per CU).  Chunks of about half a round's share keep every wavefront's
   // fixed costs (first tile, partial results, merge) small against its stream;
-  // 512 tokens is the shortest chunk worth a partial result, and beyond 2048
-  // nothing is gained (measured on 1 to 64 sequences of 32k tokens).
+  // beyond 2048 tokens nothing is gained, and the shortest chunk worth a
+  // partial result is 512 tokens, or 256 where that still leaves a sequence in
+  // no more than 32 chunks for the merge (measured on 1 to 64 sequences of 8k,
+  // 32k and 128k tokens: 1 to 4 sequences of 8k take 29 to 36 us with chunks of
+  // 256 tokens against 36 to 43 us with 512, one sequence of 32k 63 against 55).
   if (batch <= 0 || heads_kv <= 0 || max_seqlen <= 0) return 64;
   if (num_cus <= 0) num_cus = 256;
   const long long work = (long long)batch * heads_kv * max_seqlen;  // tokens x kv-heads
   long long tokens = 2 * work / (8LL * num_cus);
   tokens = (tokens + 63) / 64 * 64;
-  if (tokens < 512) tokens = 512;
+  long long shortest = (long long)max_seqlen / 32 / 64 * 64;
+  shortest = shortest < 256 ? 256 : (shortest > 512 ? 512 : shortest);
+  if (tokens < shortest) tokens = shortest;
   if (tokens > 2048) tokens = 2048;
   return (int)tokens;
 }
