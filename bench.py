@@ -144,13 +144,17 @@ def _fwd_args(q, k, v, o, lse, causal):
 DENSE_SHAPE = (4, 32, 8192, 128)
 
 
+DENSE_FORM = "auto"   # --dense-form: pin one of the two forms of the dense kernel (for profiling)
+
+
 def _dense_kernel_name(D):
-    if D == 128:
-        return KERNELS["dense_causal"]
-    name = _NS + "12dense_kernelIDF16bLi%dEEEvNS_13PrefillParamsE" % D
-    if D == 64:   # the launcher picks the form from the number of work items
-        name += " or " + KERNELS["c1_dense_noncausal_small"]
-    return name
+    long_form = _NS + "12dense_kernelIDF16bLi%dEEEvNS_13PrefillParamsE" % D
+    short_form = _NS + "18dense_short_kernelIDF16bLi%dEEEvNS_13PrefillParamsE" % D
+    if DENSE_FORM == "256" or (DENSE_FORM == "auto" and DENSE_SHAPE == (4, 32, 8192, 128)):
+        return long_form
+    if DENSE_FORM == "128":
+        return short_form
+    return long_form + " or " + short_form   # the launcher picks the form from the number of work items
 
 
 def run_dense_causal(steps, warmup):
@@ -158,10 +162,13 @@ def run_dense_causal(steps, warmup):
     B, H, S, D = DENSE_SHAPE
     q, k, v = (_randn((B, H, S, D), s) for s in (0, 1, 2))
     fn = lambda: ta.flash_attention(q, k, v, causal=True, return_lse=True)
-    ms = _time_steps(fn, steps, warmup)
+    with ta.dense_form(DENSE_FORM):
+        ms = _time_steps(fn, steps, warmup)
     o = torch.empty_like(q)
     lse = torch.empty((B, H, S), device="cuda", dtype=torch.float32)
-    kms = _event_ms(0, _fwd_args(q, k, v, o, lse, True), steps, warmup)
+    args = _fwd_args(q, k, v, o, lse, True)
+    args.dense_form = {"auto": 0, "256": 1, "128": 2}[DENSE_FORM]
+    kms = _event_ms(0, args, steps, warmup)
     flop = 2.0 * B * H * S * (S + 1) * D            # 4*D per unmasked (q, k) pair
     # parity on the benchmark tensors: three (batch, head) units x four 64-row blocks
     err = err_lse = 0.0
@@ -179,7 +186,8 @@ def run_dense_causal(steps, warmup):
         "err_sample": "o and lse of 3 (batch, head) units x 4 blocks of 64 query rows against fp32 torch math on the device",
         "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "kernel": _dense_kernel_name(D)},
-        "config": {"workload": "dense causal flash-attention fwd bf16 B=%d H=%d S=%d D=%d, o bf16 + lse fp32" % (B, H, S, D),
+        "config": {"workload": "dense causal flash-attention fwd bf16 B=%d H=%d S=%d D=%d, o bf16 + lse fp32%s"
+                               % (B, H, S, D, "" if DENSE_FORM == "auto" else ", %s-row work items" % DENSE_FORM),
                    "flop_per_step": flop, "flop_reference_convention_4BHS2D": 4.0 * B * H * S * S * D},
     }
 
@@ -1000,7 +1008,12 @@ def main():
                     help="batch, heads, sequence length and head_dim of the dense_causal workload instead of the "
                          "benchmark's 4,32,8192,128 (S a multiple of 64, at least 256; D 64, 96 or 128; for "
                          "profiling other shapes)")
+    ap.add_argument("--dense-form", default="auto", choices=["auto", "256", "128"],
+                    help="pin the dense_causal workload to one form of the dense kernel (work items of 256 or of 128 "
+                         "query rows) instead of the library's per-launch choice; for profiling")
     a = ap.parse_args()
+    global DENSE_FORM
+    DENSE_FORM = a.dense_form
     if a.dense_shape:
         global DENSE_SHAPE
         sh = tuple(int(x) for x in a.dense_shape.split(","))

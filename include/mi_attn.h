@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define MI_ATTN_ABI_VERSION 6
+#define MI_ATTN_ABI_VERSION 7
 
 /* KV tile edge (tokens) of the prefill kernels and block edge of the block
  * sparse layouts; fixed at build time. */
@@ -88,7 +88,17 @@ typedef enum mi_status {
  * cu_seqlens[batch], or behind the first max_seqlen tokens of their sequence -
  * with one small extra launch, so the caller can hand in uninitialised
  * outputs.  0 leaves such rows untouched.
+ * dense_form: the kernel comes in two forms that give the same bits - work
+ * items of 256 query rows on workgroups of eight wavefronts, one to a compute
+ * unit, and work items of 128 rows on workgroups of four wavefronts, two to a
+ * compute unit (three at head_dim 64).  MI_DENSE_FORM_AUTO lets the library
+ * pick per launch from the number of work items (the short form when every
+ * work item has a compute unit to itself; at head_dim 64 also where three
+ * workgroups per unit outrun one); the other two values are for tests and for
+ * callers who have measured their own shapes.
  */
+enum { MI_DENSE_FORM_AUTO = 0, MI_DENSE_FORM_256_ROWS = 1, MI_DENSE_FORM_128_ROWS = 2 };
+
 typedef struct mi_attn_fwd_args {
   uint32_t struct_size;
   int32_t dtype;                 /* mi_dtype of q, k, v, o                     */
@@ -107,6 +117,7 @@ typedef struct mi_attn_fwd_args {
   int32_t causal;                /* 0 / 1                                      */
   float scale_log2;              /* softmax scale * log2(e), > 0               */
   int32_t total_rows;            /* packed: rows of o / lse to cover, or 0     */
+  int32_t dense_form;            /* MI_DENSE_FORM_*                            */
 } mi_attn_fwd_args;
 
 int mi_attn_fwd(const mi_attn_fwd_args *args, void *stream);

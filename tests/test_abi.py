@@ -27,7 +27,7 @@ def test_every_declared_symbol_is_exported(lib):
     assert declared == set(_lib.EXPORTS), "ctypes table and header disagree: %s" % (declared ^ set(_lib.EXPORTS))
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.mi_abi_version() == _lib.MI_ATTN_ABI_VERSION == 6
+    assert lib.mi_abi_version() == _lib.MI_ATTN_ABI_VERSION == 7
 
 
 def test_struct_layout_matches_the_c_compiler(tmp_path):
@@ -93,6 +93,8 @@ def test_fwd_validation(lib):
         (lambda a: setattr(a, "o_stride_b", 4), "MI_ERR_STRIDE"),
         (lambda a: setattr(a, "total_rows", -1), "MI_ERR_SHAPE"),
         (lambda a: setattr(a, "total_rows", 64), "MI_ERR_SHAPE"),       # batched form: there are no rows outside the sequences
+        (lambda a: setattr(a, "dense_form", 3), "MI_ERR_SHAPE"),
+        (lambda a: setattr(a, "dense_form", -1), "MI_ERR_SHAPE"),
     ]
     for mutate, want in cases:
         a = _good_fwd()
@@ -109,6 +111,9 @@ def test_fwd_validation(lib):
     a.o_stride_b = 4
     a.total_rows = 4096
     assert lib.mi_attn_fwd_validate(C.byref(a)) == 0
+    for form in (_lib.MI_DENSE_FORM_AUTO, _lib.MI_DENSE_FORM_256_ROWS, _lib.MI_DENSE_FORM_128_ROWS):
+        a.dense_form = form
+        assert lib.mi_attn_fwd_validate(C.byref(a)) == 0
 
 
 def _good_sparse():

@@ -49,7 +49,7 @@ def dense_kernels(prefill_asm):
 @pytest.fixture(scope="module")
 def short_kernels(prefill_asm):
     kernels = _bodies(prefill_asm, "dense_short_kernel")
-    assert sorted(kernels) == [("DF16_", 64), ("DF16b", 64)], sorted(kernels)   # the short form is built for head_dim 64
+    assert len(kernels) == 6, sorted(kernels)          # bf16 / f16  x  64 / 96 / 128
     return kernels
 
 
@@ -106,34 +106,36 @@ def test_no_scratch_memory(dense_kernels, short_kernels):
         assert not any("scratch_" in l for l in lines), key
 
 
-def test_short_form_leaves_room_for_three_waves_per_simd(prefill_asm, short_kernels):
-    """Three 4-wave workgroups share a CU, one wave of each per SIMD: 512 registers
-    in allocation units of 8 leave 168 per wave.  And the item-top wait: when the
-    next item has a fourth tile its loads (one K and one V instruction per wave at
-    head_dim 64) are the youngest and may stay in flight, else everything is
-    waited for; the two arms meet in front of the barrier that opens the item."""
+def test_short_form_register_budget_and_item_top_wait(prefill_asm, short_kernels):
+    """At head_dim 64 three 4-wave workgroups share a CU, one wave of each per SIMD:
+    512 registers in allocation units of 8 leave 168 per wave.  And the item-top
+    wait of every instantiation: when the next item has a fourth tile its loads
+    (one K and one V instruction per wave at head_dim 64, two of each otherwise)
+    are the youngest and may stay in flight, else everything is waited for; the
+    two arms meet in front of the barrier that opens the item."""
     seen = 0
     for block in prefill_asm.split("- .agpr_count:")[1:]:
         kern = re.search(r"\.name:\s+(\S+)", block).group(1)
-        if "dense_short_kernel" in kern:
+        if "dense_short_kernel" in kern and "Li64E" in kern:
             assert int(re.search(r"\.vgpr_count:\s+(\d+)", block).group(1)) <= 168, kern
             seen += 1
     assert seen == 2
-    for key, lines in short_kernels.items():
-        assert len([l for l in lines if "global_store_dwordx4" in l]) == 4, key
+    for (dtype, d), lines in short_kernels.items():
+        assert len([l for l in lines if "global_store_dwordx4" in l]) == {64: 4, 96: 8, 128: 8}[d], (dtype, d)
+        tile_loads = {64: 2, 96: 4, 128: 4}[d]
         sig = _significant(lines)
         sites = []
         for k, (_, t) in enumerate(sig):
-            if t != "s_waitcnt vmcnt(2)":
+            if t != "s_waitcnt vmcnt(%d)" % tile_loads:
                 continue
             near = [j for j in range(max(0, k - 5), min(len(sig), k + 6)) if sig[j][1] == "s_waitcnt vmcnt(0)"]
             if not near:
                 continue                                  # (the waits at the top of a position also cover lgkmcnt)
             last = max(near + [k])
             nxt = next(x for _, x in sig[last + 1:] if x.startswith("s_barrier") or re.match(r"(global|buffer|scratch|flat)_", x))
-            assert nxt.startswith("s_barrier"), (key, nxt)
+            assert nxt.startswith("s_barrier"), (dtype, d, nxt)
             sites.append(k)
-        assert len(sites) == 1, (key, sites)
+        assert len(sites) == 1, (dtype, d, sites)
 
 
 def test_q_registers_are_untouched_between_load_and_wait(dense_kernels, short_kernels):

@@ -2,6 +2,7 @@
 rookie-joe/TritonOps' flash_attn_triton package."""
 from .ops import (  # noqa: F401
     LOG2E,
+    dense_form,
     flash_attention,
     flash_attention_decoding,
     flash_attention_sparse_decoding,

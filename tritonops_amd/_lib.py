@@ -9,10 +9,11 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmi_attn.so")
 
-MI_ATTN_ABI_VERSION = 6
+MI_ATTN_ABI_VERSION = 7
 MI_DECODE_STATIC_SCRATCH_BYTES = 32 << 20
 MI_KV_BATCHED, MI_KV_PACKED, MI_KV_PAGED = 0, 1, 2
 MI_ATTN_BLOCK = 64
+MI_DENSE_FORM_AUTO, MI_DENSE_FORM_256_ROWS, MI_DENSE_FORM_128_ROWS = 0, 1, 2
 MI_DTYPE_F32 = 2
 MI_DTYPE_BF16 = 0
 MI_DTYPE_F16 = 1
@@ -49,7 +50,7 @@ class AttnFwdArgs(C.Structure):
         ("cu_seqlens", _vp),
         ("batch", _i32), ("heads_q", _i32), ("heads_kv", _i32),
         ("max_seqlen", _i32), ("head_dim", _i32), ("causal", _i32),
-        ("scale_log2", _f32), ("total_rows", _i32),
+        ("scale_log2", _f32), ("total_rows", _i32), ("dense_form", _i32),
     ]
 
 

@@ -184,8 +184,10 @@ int mi_attn_fwd_validate(const mi_attn_fwd_args* a) {
   if (a->causal != 0 && a->causal != 1) return fail(MI_ERR_SHAPE, "causal must be 0 or 1");
   if (a->total_rows < 0) return fail(MI_ERR_SHAPE, "total_rows %d is negative", a->total_rows);
   if (a->total_rows > 0 && !a->cu_seqlens) return fail(MI_ERR_SHAPE, "total_rows is for the packed form (cu_seqlens != NULL)");
-  // (work item ids are 32-bit and the persistent kernel steps them by its grid size)
-  const long long wgs = (((long long)a->max_seqlen + mi::kDenseRows - 1) / mi::kDenseRows) * a->heads_q * a->batch;
+  if (a->dense_form < MI_DENSE_FORM_AUTO || a->dense_form > MI_DENSE_FORM_128_ROWS)
+    return fail(MI_ERR_SHAPE, "dense_form %d is none of MI_DENSE_FORM_AUTO / _256_ROWS / _128_ROWS", a->dense_form);
+  // (work item ids are 32-bit and the persistent kernels step them by their grid size)
+  const long long wgs = (((long long)a->max_seqlen + mi::kShortRows - 1) / mi::kShortRows) * a->heads_q * a->batch;
   if (wgs > 0x3fffffffLL) return fail(MI_ERR_SHAPE, "%lld work items are too many", wgs);
   return MI_OK;
 }
@@ -450,6 +452,7 @@ int mi_attn_fwd(const mi_attn_fwd_args* a, void* stream) {
   mi::PrefillParams p;
   fill_prefill(a, p, mi::kDenseRows);
   p.causal = a->causal;
+  p.dense_form = a->dense_form;
   return launch_status(mi::launch_prefill_dense(p, a->dtype, a->head_dim, static_cast<hipStream_t>(stream)), "mi_attn_fwd");
 }
 

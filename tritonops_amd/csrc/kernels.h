@@ -26,6 +26,7 @@ struct PrefillParams {
   int32_t n_qtiles;  // ceil(max_seqlen / rows per workgroup)
   int32_t n_items;   // logical workgroups = n_qtiles * hq * batch (set by the launcher)
   int32_t causal;
+  int32_t dense_form;             // dense only: 0 chosen per launch, 1 256-row items, 2 128-row items
   int32_t win_local, win_global;  // -1 => off
   float scale;                    // log2 domain
 };
@@ -197,12 +198,14 @@ int launch_xent_dlogits(const XentGradParams& p, int dtype, hipStream_t s);
 // Query rows per workgroup of the two prefill kernels.
 constexpr int kDenseRows = 256;
 constexpr int kSparseRows = 64;
-// The short form of the dense kernel (head_dim 64): query rows per workgroup,
-// LDS stages, keys per tile, workgroups resident per CU.
+// The short form of the dense kernel: query rows per workgroup, LDS stages,
+// keys per tile, workgroups resident per CU (three at head_dim 64, whose waves
+// need 163 registers; two otherwise).
 constexpr int kShortRows = 128;
 constexpr int kShortStages = 5;
 constexpr int kShortTileKeys = 32;
 constexpr int kShortPerCu = 3;
+constexpr int short_per_cu(int head_dim) { return head_dim == 64 ? kShortPerCu : 2; }
 // LDS stages of the two prefill kernels: KV tiles resident per workgroup
 // (dense), K tiles and V tiles resident per workgroup (block-sparse: the K
 // ring runs one tile ahead of the V ring).

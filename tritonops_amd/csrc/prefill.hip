@@ -1158,25 +1158,30 @@ dense_kernel(const PrefillParams p) {
 }
 
 // ---------------------------------------------------------------------------
-// Dense, short form (head_dim 64): workgroups of 4 wavefronts (128 query rows
-// per item), three to a CU, KV tiles of 32 keys in a ring of five stages
-// (40 KiB of LDS per workgroup at head_dim 64).
+// Dense, short form: workgroups of 4 wavefronts (128 query rows per item), KV
+// tiles of 32 keys in a ring of five stages (80 KiB of LDS per workgroup, 40 at
+// head_dim 64), two workgroups to a CU, three at head_dim 64.
 //
-// dense_kernel keeps one 8-wave workgroup per CU, two wavefronts per SIMD.  At
-// head_dim 64 the softmax arithmetic outweighs the matrix work (56 vector
-// instructions against 8 MFMAs per 32 x 32 block of scores) and a wave's
-// registers (O, S, Q^T, P: 163 in all) leave room for a third wavefront per
-// SIMD, which fills issue slots that two leave empty; three independent
-// workgroups also run one another's item boundaries under their tile loops.
-// Measured against dense_kernel at head_dim 64 (HIP events, same box): 3 to 8 %
-// faster on launches of eight rounds or more (4 x 8192 tokens, 32 heads: 1158
-// against 1190 us), 6 to 11 % on 16 sequences of 2048 / 512 tokens, 4 to 10 % on
-// launches of at most one workgroup per CU; slower where the item count is a
-// round and a bit (1024 items on 768 slots) while dense_kernel's rounds come
-// out even, which the launcher works out per launch (short_form_pays).  At head_dim 96 and 128 a wave needs 185 / 218 registers, two
-// fit a SIMD either way, and this form measured equal or slower: it is built
-// for head_dim 64 only.  The price is twice the tile traffic from the L2s per
-// query row.
+// dense_kernel keeps one 8-wave workgroup per CU, two wavefronts per SIMD, and
+// a work item is one chain of latencies (geometry, Q and first tiles, the exact
+// first half, the tile loop, normalise, stage, store).  Two uses:
+//  - launches with at most one 128-row item per CU (short prompts, few heads):
+//    twice as many CUs work, each on a chain half as long.  10 to 17 % faster
+//    than dense_kernel at head_dim 128 on every such launch measured (1 to 4
+//    sequences of 256 to 4096 tokens, 8 and 32 heads, causal and not); with
+//    more items than CUs the two forms are within 5 % of each other at head_dim
+//    96 and 128 (two waves per SIMD either way) and dense_kernel stays ahead.
+//  - head_dim 64: the softmax arithmetic outweighs the matrix work there (56
+//    vector instructions against 8 MFMAs per 32 x 32 block of scores) and a
+//    wave's registers (O, S, Q^T, P: 163 in all) leave room for a third
+//    wavefront per SIMD, which fills issue slots that two leave empty.  3 to 8 %
+//    faster than dense_kernel on launches of eight rounds or more (4 x 8192
+//    tokens, 32 heads: 1158 against 1190 us), 6 to 11 % on 16 sequences of 2048
+//    / 512 tokens; slower where the item count is a round and a bit (1024 items
+//    on 768 slots) while dense_kernel's rounds come out even, which the launcher
+//    works out per launch (short_form_pays).
+// The price is twice the tile traffic from the L2s per query row.
+//
 //
 // The same half-tile software pipeline as dense_kernel, a tile now being one
 // half: at position h a wave forms S(h+1) = K(h+1) Q^T together with the second
@@ -1189,7 +1194,7 @@ dense_kernel(const PrefillParams p) {
 // alternate with the position's parity and the ring has five stages, so the
 // tile loop is unrolled ten times.
 template <typename T, int D>
-__global__ void __launch_bounds__(kShortRows * 2) __attribute__((amdgpu_waves_per_eu(kShortPerCu)))
+__global__ void __launch_bounds__(kShortRows * 2) __attribute__((amdgpu_waves_per_eu(short_per_cu(D))))
 dense_short_kernel(const PrefillParams p) {
   constexpr int NW = kShortRows / 32, NS = kShortStages, TN = kShortTileKeys;
   static_assert(NW == 4 && NS == 5 && TN == 32, "stage use at the item boundary assumes this shape");
@@ -1598,24 +1603,32 @@ template <typename T, int D>
 int launch_short(const PrefillParams& p, long long items, int cus, hipStream_t s) {
   auto kern = dense_short_kernel<T, D>;
   constexpr size_t lds = prefill_lds_bytes<D, kShortRows / 32, kShortStages, kShortTileKeys>();
-  static_assert(kShortPerCu * lds <= 160 * 1024, "kShortPerCu workgroups share a CU's LDS");
+  constexpr int per_cu = short_per_cu(D);
+  static_assert(per_cu * lds <= 160 * 1024, "that many workgroups share a CU's LDS");
   static LdsLimitOnce lds_once;
   if (const int e = raise_lds_limit(lds_once, reinterpret_cast<const void*>(kern), (int)lds)) return e;
   PrefillParams pp = p;
   pp.n_qtiles = (p.max_seqlen + kShortRows - 1) / kShortRows;
   pp.n_items = (int)items;
   long long grid = items;
-  if (grid > (long long)kShortPerCu * cus) grid = (long long)kShortPerCu * cus;
+  if (cus > 0 && grid > (long long)per_cu * cus) grid = (long long)per_cu * cus;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kShortRows * 2), lds, s, pp);
   return (int)hipGetLastError();
 }
 
 template <typename T, int D, bool SPARSE>
 int launch_one(const PrefillParams& p, hipStream_t s) {
-  if constexpr (!SPARSE && D == 64) {
+  if constexpr (!SPARSE) {
     const int cus = device_cu_count();
     const long long n = (long long)((p.max_seqlen + kShortRows - 1) / kShortRows) * p.hq * p.batch;
-    if (short_form_pays(n, (long long)p.n_qtiles * p.hq * p.batch, cus)) return launch_short<T, D>(p, n, cus, s);
+    bool short_form = p.dense_form == 2;
+    if (p.dense_form == 0) {
+      if (D == 64)
+        short_form = short_form_pays(n, (long long)p.n_qtiles * p.hq * p.batch, cus);
+      else
+        short_form = cus > 0 && n <= cus;   // a CU per 128-row item
+    }
+    if (short_form) return launch_short<T, D>(p, n, cus, s);
   }
   constexpr int NW = (SPARSE ? kSparseRows : kDenseRows) / 32;
   constexpr int NS = SPARSE ? kSparseStages : kDenseStages;

@@ -5,8 +5,10 @@ Names, positional arguments and semantics follow the reference launchers
 is done by the HIP kernels of libmi_attn.so reached through its C ABI.  There
 is no fallback: without the built library every call raises.
 """
+import contextlib
 import ctypes as C
 import math
+import threading
 import weakref
 
 import torch
@@ -132,6 +134,27 @@ def _fill_qkvo(a, q, k, v, o, lse, packed):
         a.lse_stride_h = lse.stride(2)
 
 
+_DENSE_FORMS = {"auto": _lib.MI_DENSE_FORM_AUTO, "256": _lib.MI_DENSE_FORM_256_ROWS, "128": _lib.MI_DENSE_FORM_128_ROWS}
+_dense_form = threading.local()
+
+
+@contextlib.contextmanager
+def dense_form(form):
+    """Dense forward calls of this thread inside the block run in one form of
+    the kernel: "256" (work items of 256 query rows, 8-wave workgroups), "128"
+    (128 rows, 4-wave workgroups) or "auto" (the library picks per launch, the
+    default).  The forms give the same bits; the switch is for tests and for
+    callers who have timed their own shapes."""
+    if form not in _DENSE_FORMS:
+        raise ValueError("dense_form takes 'auto', '256' or '128', got %r" % (form,))
+    before = getattr(_dense_form, "value", _lib.MI_DENSE_FORM_AUTO)
+    _dense_form.value = _DENSE_FORMS[form]
+    try:
+        yield
+    finally:
+        _dense_form.value = before
+
+
 def _dense_fwd(q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, want_lse=True, bhsd=False):
     """q,k,v as [X, S, H, D] (see _fill_qkvo). Returns (o, lse[X, S, H]); with
     `bhsd` the outputs own [X, H, S, D] / [X, H, S] memory and are returned as
@@ -180,6 +203,7 @@ def _dense_fwd(q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, want_lse=T
     a.heads_q, a.heads_kv, a.head_dim = Hq, k.shape[2], D
     a.causal = 1 if causal else 0
     a.scale_log2 = float(scale_log2)
+    a.dense_form = getattr(_dense_form, "value", _lib.MI_DENSE_FORM_AUTO)
     _lib.check(lib.mi_attn_fwd(C.byref(a), _stream()))
     return o, lse
 
