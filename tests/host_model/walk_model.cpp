@@ -465,7 +465,7 @@ static void test(std::mt19937& rng) {
         ++cases;
       }
     }
-    // the short form of the same kernel (head_dim 64): 128-row items, three workgroups per CU
+    // the short form of the same kernel: 128-row items, two or three workgroups per CU
     {
       const int nq = (s.max_seqlen + short_form::BM - 1) / short_form::BM;
       const int ni = nq * s.hq * s.batch;
