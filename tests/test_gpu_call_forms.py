@@ -95,6 +95,44 @@ def test_python_forms_return_zero_rows_outside_the_sequences():
     assert_close(os_[:, :used], want, TOL, "window-sparse o")
 
 
+def test_zeroing_follows_what_the_host_knows_about_cu_seq_lens():
+    """When the host has read a cu_seq_lens tensor and its sequences tile the whole
+    buffer, the drop-ins skip the launch that zeroes rows outside the sequences;
+    an in-place change of that tensor, a max_seq_len below the longest sequence,
+    or a first entry above 0 must bring it back."""
+    import tritonops_amd as ta
+    from tritonops_amd import ops
+
+    T, Hq, Hkv, D = 512, 4, 2, 64
+    q, k, v = (randn((1, T, h, D), s).cuda() for s, h in ((1, Hq), (2, Hkv), (3, Hkv)))
+    cu = torch.tensor([0, 200, 512], dtype=torch.int32, device="cuda")
+
+    def dirty():
+        for _ in range(4):
+            junk = torch.full((T * Hq * D,), SENTINEL, device="cuda", dtype=torch.float32)
+            del junk
+
+    dirty()
+    o, lse = ta.flash_attention(q, k, v, cu, return_lse=True)          # reads the lengths on the host
+    assert ops._rows_to_cover(cu, 312, T) == 0 and ops._rows_to_cover(cu, 311, T) == T
+    want = orc.flash_attn_torch(q.cpu(), k.cpu(), v.cpu(), cu.cpu(), faithful=False)
+    assert_close(o, want, TOL, "o, every row inside a sequence")
+    o2 = ta.flash_attention(q, k, v, cu, max_seq_len=100)             # both sequences cut: rows behind token 100 are zero
+    assert (o2[:, 100:200] == 0).all() and (o2[:, 300:] == 0).all()
+    assert_close(o2[:, :100], want[:, :100], TOL, "kept rows")
+    cu[2] = 400                                                        # in place: the version counter moves
+    dirty()
+    o3, lse3 = ta.flash_attention(q, k, v, cu, return_lse=True)
+    assert (o3[:, 400:] == 0).all() and (lse3[:, 400:] == 0).all()
+    assert ops._rows_to_cover(cu, 512, T) == T
+    cu2 = torch.tensor([64, 200, 512], dtype=torch.int32, device="cuda")   # rows in front of the first sequence
+    dirty()
+    o4 = ta.flash_attention(q, k, v, cu2)
+    assert (o4[:, :64] == 0).all()
+    os_, ls = ta.flash_attn_sparse_triton(q, k, v, cu, None, 64, 64)
+    assert (os_[:, 400:] == 0).all() and (ls[:, 400:] == 0).all()
+
+
 def test_max_seqlen_below_the_longest_sequence_cuts_it():
     """A bound smaller than a real length must not write outside what was sized
     for it: the long sequence is cut at the bound (for a causal forward the kept

@@ -62,30 +62,54 @@ def _ptr(t):
     return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
 
 
-_MAX_LEN_CACHE = {}   # id(cu tensor) -> (weak reference, version counter, longest sequence)
+_MAX_LEN_CACHE = {}   # id(cu tensor) -> (weak reference, version counter, longest sequence, first and last entry)
+
+
+def _cu_facts(cu_seq_lens):
+    """(longest sequence, cu[0], cu[-1]) of a cu_seq_lens tensor, kept per tensor
+    OBJECT for as long as that object lives and its version counter (bumped by
+    every in-place write) has not moved; one host round trip the first time."""
+    key = id(cu_seq_lens)
+    hit = _MAX_LEN_CACHE.get(key)
+    if hit is not None and hit[0]() is cu_seq_lens and hit[1] == cu_seq_lens._version:
+        return hit[2]
+    if cu_seq_lens.numel() < 2:
+        facts = (0, 0, 0)
+    else:
+        facts = tuple(int(x) for x in torch.stack(
+            [(cu_seq_lens[1:] - cu_seq_lens[:-1]).max(), cu_seq_lens[0], cu_seq_lens[-1]]).tolist())
+    if len(_MAX_LEN_CACHE) >= 256:
+        _MAX_LEN_CACHE.clear()
+    try:
+        _MAX_LEN_CACHE[key] = (weakref.ref(cu_seq_lens), cu_seq_lens._version, facts)
+    except TypeError:
+        pass
+    return facts
 
 
 def _max_len(cu_seq_lens, max_seq_len):
     """Longest sequence of the batch, which sizes the launch.  Without a hint
     it costs the host round trip the reference launcher makes on every call
     (flash_attn_triton/flash_attn_triton.py:621); here the answer is kept per
-    cu_seq_lens tensor OBJECT for as long as that object lives and its version
-    counter (bumped by every in-place write) has not moved, so the layers of a
-    model that share one cu_seq_lens pay for it once per batch."""
+    cu_seq_lens tensor object (_cu_facts), so the layers of a model that share
+    one cu_seq_lens pay for it once per batch."""
     if max_seq_len is not None:
         return int(max_seq_len)
-    key = id(cu_seq_lens)
-    hit = _MAX_LEN_CACHE.get(key)
-    if hit is not None and hit[0]() is cu_seq_lens and hit[1] == cu_seq_lens._version:
-        return hit[2]
-    n = int((cu_seq_lens[1:] - cu_seq_lens[:-1]).max().item())
-    if len(_MAX_LEN_CACHE) >= 256:
-        _MAX_LEN_CACHE.clear()
-    try:
-        _MAX_LEN_CACHE[key] = (weakref.ref(cu_seq_lens), cu_seq_lens._version, n)
-    except TypeError:
-        pass
-    return n
+    return _cu_facts(cu_seq_lens)[0]
+
+
+def _rows_to_cover(cu_seq_lens, max_seqlen, rows):
+    """total_rows of a packed call: `rows` (the library zeroes the rows of the
+    outputs that belong to no sequence), or 0 when the host already knows that
+    there is no such row - the sequences tile [0, rows) and none is longer than
+    the `max_seqlen` the call runs with - which saves the small launch that
+    looks for them.  Known only while the lengths of this cu_seq_lens object
+    are on file from an earlier host read (_cu_facts); never read here."""
+    hit = _MAX_LEN_CACHE.get(id(cu_seq_lens))
+    if hit is None or hit[0]() is not cu_seq_lens or hit[1] != cu_seq_lens._version:
+        return rows
+    longest, first, last = hit[2]
+    return 0 if (first == 0 and last == rows and longest <= max_seqlen) else rows
 
 
 _HEAD_DIMS = (64, 96, 128)
@@ -201,7 +225,7 @@ def _dense_fwd(q, k, v, cu_seq_lens, scale_log2, causal, max_seq_len, want_lse=T
         a.cu_seqlens = _ptr(cu)
         a.batch = cu.numel() - 1
         a.max_seqlen = min(_max_len(cu_seq_lens, max_seq_len), S)
-        a.total_rows = S
+        a.total_rows = _rows_to_cover(cu_seq_lens, a.max_seqlen, S)
     else:
         a.cu_seqlens = None
         a.batch = X
@@ -252,7 +276,7 @@ def _dense_bwd(q, k, v, o, do, lse, cu_seq_lens, scale_log2, causal, max_seq_len
         a.cu_seqlens = _ptr(cu)
         a.batch = cu.numel() - 1
         a.max_seqlen = min(_max_len(cu_seq_lens, max_seq_len), S)
-        a.total_rows = S  # rows outside every sequence receive zeros
+        a.total_rows = _rows_to_cover(cu_seq_lens, a.max_seqlen, S)  # rows outside every sequence receive zeros
     else:
         a.cu_seqlens = None
         a.batch = X
@@ -456,7 +480,7 @@ def flash_attn_sparse_triton(q, k, v, cu_seqlens, softmax_scale=None, local_wind
     a.block_size = _masks.BLOCK
     a.window_local, a.window_global = wl, wg
     a.scale_log2 = scale
-    a.total_rows = T if packed else 0
+    a.total_rows = _rows_to_cover(cu_seqlens, max_len, T) if packed else 0
     _lib.check(lib.mi_attn_fwd_blocksparse(C.byref(a), _stream()))
     return o, lse
 
