@@ -509,12 +509,11 @@ template <typename T, int D>
 __device__ __forceinline__ void bwd_dkdv_item(const BwdParams& p, const int bid, const int n_rt) {
   using G = RowGeom<D>;
   using F = UniFrags<D>;
-  constexpr int NW = 8, NP = 4, BM = 32 * NP, TN = 64, NS = kBwdStages;
+  constexpr int NP = 4, BM = 32 * NP, TN = 64, NS = kBwdStages;
   static_assert(NS == 3, "stage reuse below assumes three stages");
   constexpr int TILEB = TN * F::ROWB;
   constexpr int STAGEB = 2 * TILEB + 1024;
   constexpr int RPI = 1024 / F::ROWB;
-  constexpr int IPW = TN / RPI / NW;
   constexpr int OROWB = D * 2 + 16;
   constexpr uint32_t PBUF = NS * STAGEB;       // P exchange: [2 tile slots][NP pairs][2 blocks][2 KiB]
   constexpr uint32_t PSLOT = NP * 2 * 2048;

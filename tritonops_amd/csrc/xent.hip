@@ -85,13 +85,6 @@ __global__ void __launch_bounds__(512) xent_gemm_kernel(const XentParams p) {
   const int total = tile_cnt * nk;
 
   const uint32_t lds0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)xsmem);
-  auto dma16 = [&](uint64_t g, uint32_t slab_u) __attribute__((always_inline)) {
-    const uint32_t slab = (uint32_t)__builtin_amdgcn_readfirstlane(slab_u);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                 :
-                 : "v"(g), "s"(slab)
-                 : "memory");
-  };
   auto uniform64 = [](uint64_t v) __attribute__((always_inline)) -> uint64_t {
     const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)v);
     const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
