@@ -485,6 +485,29 @@ def test_window_csr_is_built_once():
     assert (a[0] == want[0]).all() and (a[1] == want[1]).all() and a[2] == want[2]
 
 
+def test_host_knowledge_of_cu_seq_lens_follows_the_tensor():
+    """The drop-ins keep what one host read of a cu_seq_lens tensor told them (longest
+    sequence, first and last entry) for as long as that tensor object is unmodified, and
+    decide from it whether any row of a packed output lies outside every sequence."""
+    import torch
+
+    from tritonops_amd import ops
+
+    cu = torch.tensor([0, 200, 512], dtype=torch.int32)
+    assert ops._rows_to_cover(cu, 512, 512) == 512          # nothing on file yet: the library looks for such rows
+    assert ops._max_len(cu, None) == 312                    # the host read
+    assert ops._rows_to_cover(cu, 312, 512) == 0            # the sequences tile [0, 512) and none is cut
+    assert ops._rows_to_cover(cu, 311, 512) == 512          # the longer sequence would be cut
+    assert ops._rows_to_cover(cu, 312, 600) == 600          # padding rows behind the last sequence
+    assert ops._max_len(cu, 100) == 100                     # a hint is taken as it is
+    cu[2] = 400                                             # in place: the version counter moves
+    assert ops._rows_to_cover(cu, 512, 512) == 512
+    assert ops._max_len(cu, None) == 200 and ops._rows_to_cover(cu, 200, 400) == 0
+    lead = torch.tensor([64, 200, 512], dtype=torch.int32)
+    assert ops._max_len(lead, None) == 312 and ops._rows_to_cover(lead, 312, 512) == 512   # rows in front of the first sequence
+    assert ops._max_len(torch.tensor([0], dtype=torch.int32), None) == 0
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     """No fallback: with the shared library absent every entry point raises."""
     import torch
