@@ -40,7 +40,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 _NS = "_ZN2mi12_GLOBAL__N_1"
 KERNELS = {
     "dense_causal": _NS + "12dense_kernelIDF16bLi128EEEvNS_13PrefillParamsE",
-    "c1_dense_noncausal_small": _NS + "18dense_short_kernelIDF16bLi64EEEvNS_13PrefillParamsE",
+    "c1_dense_noncausal_small": _NS + "18dense_short_kernelIDF16bLi64ELb0EEEvNS_13PrefillParamsE",
     "gqa_decode": _NS + "21decode_splitkv_kernelIDF16bLi128EEEvNS_12DecodeParamsE",
     "block_sparse": _NS + "13sparse_kernelIDF16bLi128EEEvNS_13PrefillParamsE",
     "sparse_decode": _NS + "21decode_splitkv_kernelIDF16bLi128EEEvNS_12DecodeParamsE",
@@ -149,7 +149,7 @@ DENSE_FORM = "auto"   # --dense-form: pin one of the two forms of the dense kern
 
 def _dense_kernel_name(D):
     long_form = _NS + "12dense_kernelIDF16bLi%dEEEvNS_13PrefillParamsE" % D
-    short_form = _NS + "18dense_short_kernelIDF16bLi%dEEEvNS_13PrefillParamsE" % D
+    short_form = _NS + "18dense_short_kernelIDF16bLi%dELb0EEEvNS_13PrefillParamsE" % D
     if DENSE_FORM == "256" or (DENSE_FORM == "auto" and DENSE_SHAPE == (4, 32, 8192, 128)):
         return long_form
     if DENSE_FORM == "128":

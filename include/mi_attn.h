@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define MI_ATTN_ABI_VERSION 7
+#define MI_ATTN_ABI_VERSION 8
 
 /* KV tile edge (tokens) of the prefill kernels and block edge of the block
  * sparse layouts; fixed at build time. */
@@ -183,6 +183,15 @@ int mi_attn_bwd(const mi_attn_bwd_args *args, void *stream);
  * window is applied on top of the block list inside every live block:
  *   allowed(q,k) = k <= q and (q - k < window_local or k < window_global).
  * Pass -1 / -1 for a pure block mask.
+ * The window form needs no lists: with row_ptr = col_idx = NULL (both), and
+ * window_local >= 1 and window_global >= 0, the blocks follow from the two
+ * windows (the reference's launcher takes nothing else, :237-326): every 128
+ * query rows walk the tiles of the first window_global keys and the band of
+ * tiles that ends at their diagonal, on the dense kernel's pipeline.  Same
+ * results as the call with the window's lists up to summation order; faster
+ * than it for local windows of 2048 tokens or more at head_dim 96 / 128,
+ * slower for short windows and at head_dim 64 (the lists are then the better
+ * call).  window_local = 0 (not even the diagonal is visible) takes lists.
  * A query row with no allowed key yields o = 0 and lse = -inf.
  * total_rows as in mi_attn_fwd (the reference launcher zero-fills both outputs,
  * flash_attn_sparse_attn_triton.py:274-275).
@@ -199,8 +208,8 @@ typedef struct mi_attn_sparse_args {
   int64_t o_stride_b, o_stride_s, o_stride_h;
   int64_t lse_stride_b, lse_stride_s, lse_stride_h;
   const int32_t *cu_seqlens;     /* device [batch+1] or NULL (batched)         */
-  const int32_t *row_ptr;        /* device [n_q_blocks+1] per (b,h) slice      */
-  const int32_t *col_idx;        /* device                                     */
+  const int32_t *row_ptr;        /* device [n_q_blocks+1] per (b,h) slice, or  */
+  const int32_t *col_idx;        /* device; both NULL: the window form         */
   int64_t row_ptr_stride_b, row_ptr_stride_h;
   int64_t col_idx_stride_b, col_idx_stride_h;
   int32_t batch, heads_q, heads_kv;

@@ -27,7 +27,7 @@ def test_every_declared_symbol_is_exported(lib):
     assert declared == set(_lib.EXPORTS), "ctypes table and header disagree: %s" % (declared ^ set(_lib.EXPORTS))
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.mi_abi_version() == _lib.MI_ATTN_ABI_VERSION == 7
+    assert lib.mi_abi_version() == _lib.MI_ATTN_ABI_VERSION == 8
 
 
 def test_struct_layout_matches_the_c_compiler(tmp_path):
@@ -144,6 +144,13 @@ def test_sparse_validation(lib):
         rc = lib.mi_attn_fwd_blocksparse_validate(C.byref(a))
         assert lib.mi_status_name(rc).decode() == want
         assert lib.mi_attn_fwd_blocksparse(C.byref(a), None) == rc
+    # no lists at all: the token-window form, which needs both windows and a local one of at least a token
+    a = _good_sparse()
+    a.row_ptr = a.col_idx = None
+    for wl, wg, rc in ((-1, -1, -1), (0, 64, -1), (1, 0, 0), (4096, 128, 0), (2 ** 31 - 1, 2 ** 31 - 1, 0)):
+        a.window_local, a.window_global = wl, wg
+        assert lib.mi_attn_fwd_blocksparse_validate(C.byref(a)) == rc, (wl, wg)
+        assert rc == 0 or "window_local >= 1" in _err(lib)
 
 
 def _good_decode():

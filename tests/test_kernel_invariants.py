@@ -31,9 +31,13 @@ def prefill_asm(tmp_path_factory):
     return out.read_text()
 
 
-def _bodies(text, family):
+def _bodies(text, family, flag=None):
+    """{(dtype, head_dim): lines} of the instantiations of a kernel template; `flag` picks the
+    value of a third, boolean template argument where the template has one."""
     kernels = {}
-    for m in re.finditer(r"^(_ZN2mi\S*\d%sI(\S+?)Li(\d+)E\S*):" % family, text, re.M):
+    for m in re.finditer(r"^(_ZN2mi\S*\d%sI(\S+?)Li(\d+)E(?:Lb([01])E)?\S*):" % family, text, re.M):
+        if m.group(4) != flag:
+            continue
         body = text[m.end():text.index("s_endpgm", m.end())]
         kernels[(m.group(2), int(m.group(3)))] = body.split("\n")
     return kernels
@@ -48,8 +52,13 @@ def dense_kernels(prefill_asm):
 
 @pytest.fixture(scope="module")
 def short_kernels(prefill_asm):
-    kernels = _bodies(prefill_asm, "dense_short_kernel")
+    """The dense walk (dense_short_kernel<T, D, false>) and, under dtype + "/window", the same
+    kernel walking the tiles of a token window (dense_short_kernel<T, D, true>): one protocol."""
+    kernels = _bodies(prefill_asm, "dense_short_kernel", "0")
     assert len(kernels) == 6, sorted(kernels)          # bf16 / f16  x  64 / 96 / 128
+    window = _bodies(prefill_asm, "dense_short_kernel", "1")
+    assert len(window) == 6, sorted(window)
+    kernels.update({(dtype + "/window", d): lines for (dtype, d), lines in window.items()})
     return kernels
 
 
@@ -119,7 +128,7 @@ def test_short_form_register_budget_and_item_top_wait(prefill_asm, short_kernels
         if "dense_short_kernel" in kern and "Li64E" in kern:
             assert int(re.search(r"\.vgpr_count:\s+(\d+)", block).group(1)) <= 168, kern
             seen += 1
-    assert seen == 2
+    assert seen == 4                                   # bf16 / f16  x  dense / window
     for (dtype, d), lines in short_kernels.items():
         assert len([l for l in lines if "global_store_dwordx4" in l]) == {64: 4, 96: 8, 128: 8}[d], (dtype, d)
         tile_loads = {64: 2, 96: 4, 128: 4}[d]

@@ -9,7 +9,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmi_attn.so")
 
-MI_ATTN_ABI_VERSION = 7
+MI_ATTN_ABI_VERSION = 8
 MI_DECODE_STATIC_SCRATCH_BYTES = 32 << 20
 MI_KV_BATCHED, MI_KV_PACKED, MI_KV_PAGED = 0, 1, 2
 MI_ATTN_BLOCK = 64

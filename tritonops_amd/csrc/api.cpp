@@ -464,12 +464,17 @@ int mi_attn_fwd_blocksparse_validate(const mi_attn_sparse_args* a) {
   if (rc) return rc;
   if ((rc = check_qkvo(a))) return rc;
   if ((rc = check_prefill_strides(a))) return rc;
-  if (!a->row_ptr || !a->col_idx) return fail(MI_ERR_NULL_POINTER, "row_ptr and col_idx must be non-NULL");
+  if ((a->row_ptr == nullptr) != (a->col_idx == nullptr))
+    return fail(MI_ERR_NULL_POINTER, "row_ptr and col_idx must both be given or both be NULL");
   if (a->block_size != MI_ATTN_BLOCK) return fail(MI_ERR_SPARSE_LAYOUT, "block_size %d must be %d", a->block_size, MI_ATTN_BLOCK);
   if (a->row_ptr_stride_b < 0 || a->row_ptr_stride_h < 0 || a->col_idx_stride_b < 0 || a->col_idx_stride_h < 0)
     return fail(MI_ERR_SPARSE_LAYOUT, "mask strides must be >= 0");
   if ((a->window_local < 0) != (a->window_global < 0) || a->window_local < -1 || a->window_global < -1)
     return fail(MI_ERR_SPARSE_LAYOUT, "window_local/window_global must both be -1 or both be >= 0");
+  // no lists: the token-window form, whose blocks follow from the two windows
+  if (!a->row_ptr && (a->window_local < 1 || a->window_global < 0))
+    return fail(MI_ERR_NULL_POINTER, "without row_ptr / col_idx the call needs window_local >= 1 and window_global >= 0 (got %d, %d)",
+                a->window_local, a->window_global);
   if (a->total_rows < 0) return fail(MI_ERR_SHAPE, "total_rows %d is negative", a->total_rows);
   if (a->total_rows > 0 && !a->cu_seqlens) return fail(MI_ERR_SHAPE, "total_rows is for the packed form (cu_seqlens != NULL)");
   const long long wgs = (((long long)a->max_seqlen + mi::kSparseRows - 1) / mi::kSparseRows) * a->heads_q * a->batch;
@@ -483,6 +488,13 @@ int mi_attn_fwd_blocksparse(const mi_attn_sparse_args* a, void* stream) {
   if ((rc = zero_uncovered(a, static_cast<hipStream_t>(stream)))) return rc;
   if (a->max_seqlen == 0) return MI_OK;
   mi::PrefillParams p;
+  if (!a->row_ptr) {
+    fill_prefill(a, p, mi::kShortRows);
+    p.causal = 1;
+    // (a window as long as the longest sequence already is the whole sequence)
+    p.win_local = std::min(a->window_local, a->max_seqlen); p.win_global = std::min(a->window_global, a->max_seqlen);
+    return launch_status(mi::launch_prefill_window(p, a->dtype, a->head_dim, static_cast<hipStream_t>(stream)), "mi_attn_fwd_blocksparse");
+  }
   fill_prefill(a, p, mi::kSparseRows);
   p.causal = 1;
   p.row_ptr = a->row_ptr; p.col_idx = a->col_idx;

@@ -171,6 +171,9 @@ int launch_zero_uncovered_rows(const RowFillParams& p, hipStream_t s);
 // dtype: 0 bf16, 1 f16.  head_dim in {64, 96, 128}.  Return hipError_t as int.
 int launch_prefill_dense(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);
 int launch_prefill_sparse(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);
+// token-window form without block lists (win_local >= 1, win_global >= 0, causal): the 128-row form of the
+// dense walk over the sink tiles and the band of each item
+int launch_prefill_window(const PrefillParams& p, int dtype, int head_dim, hipStream_t s);
 int launch_decode_splitkv(const DecodeParams& p, int dtype, int head_dim, hipStream_t s);
 int launch_decode_merge(const DecodeParams& p, int dtype, int head_dim, hipStream_t s);
 // Bytes of the static device buffer behind mi_decode_noalloc

@@ -1195,7 +1195,17 @@ dense_kernel(const PrefillParams p) {
 // be in flight (counted wait, loads retire in issue order).  Score registers
 // alternate with the position's parity and the ring has five stages, so the
 // tile loop is unrolled ten times.
-template <typename T, int D>
+//
+// WIN: the token-window form (causal, key > query - win_local or key <
+// win_global) without block lists.  The keys a 128-row item can see are the
+// tiles of the first win_global keys (the sink tiles) and a band of tiles that
+// ends at its diagonal block, so the walk is the dense one over a shorter
+// sequence of tiles: position j is tile j when j < n_sink and tile j + skip
+// otherwise.  The window's lower edge is masked per key like the diagonal.
+// With win_global == 0 the first positions of an item lie below the window of
+// its later rows: a row that has not met a visible key has no reference point
+// yet and takes the exact path until it has one.
+template <typename T, int D, bool WIN>
 __global__ void __launch_bounds__(kShortRows * 2) __attribute__((amdgpu_waves_per_eu(short_per_cu(D))))
 dense_short_kernel(const PrefillParams p) {
   constexpr int NW = kShortRows / 32, NS = kShortStages, TN = kShortTileKeys;
@@ -1218,12 +1228,18 @@ dense_short_kernel(const PrefillParams p) {
 
   struct Item {
     int len, q0, n_tiles;
+    int n_sink, skip;  // WIN: positions below n_sink are tiles of their own number, the others lie `skip` tiles further on
     const T* qp;
     T* op;
     float* lp;
     KvSrc<T> kv;
   };
+  // first key of the tile at position j of an item's walk
+  auto key_of = [](const Item& it, int j) __attribute__((always_inline)) -> int {
+    return WIN ? (j + (j >= it.n_sink ? it.skip : 0)) * TN : j * TN;
+  };
   const int grid = gridDim.x;
+  const int wl = p.win_local, wg = p.win_global;
   int round = 0, base = 0;
   auto next_item = [&](Item& it) __attribute__((always_inline)) -> bool {
     while (base < p.n_items) {
@@ -1238,6 +1254,13 @@ dense_short_kernel(const PrefillParams p) {
         it.q0 = g.qt * BM;
         it.n_tiles = (g.len + TN - 1) / TN;
         if (causal) it.n_tiles = min(it.n_tiles, (it.q0 + BM + TN - 1) / TN);
+        it.n_sink = it.skip = 0;
+        if (WIN) {
+          const int t0 = max(it.q0 - wl + 1, 0) / TN;  // tile of the first key inside the local window of the item's first row
+          it.n_sink = min((wg + TN - 1) / TN, t0);
+          it.skip = t0 - it.n_sink;
+          it.n_tiles -= it.skip;
+        }
         it.qp = reinterpret_cast<const T*>(p.q) + g.q_off + g.h * p.q_sh;
         it.op = reinterpret_cast<T*>(p.o) + g.o_off + g.h * p.o_sh;
         it.lp = p.lse ? p.lse + g.lse_off + g.h * p.lse_sh : nullptr;
@@ -1256,11 +1279,11 @@ dense_short_kernel(const PrefillParams p) {
 #pragma unroll
     for (int c = 0; c < G::KSTEPS; ++c)
       asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(Q[c]) : "v"(qr), "n"(32 * c));
-    if (0 < it.n_tiles) dma.template tile<0>(it.kv, 0);
+    if (0 < it.n_tiles) dma.template tile<0>(it.kv, key_of(it, 0));
   };
   auto request_tile = [&](auto j_c, const Item& it) __attribute__((always_inline)) {
     constexpr int J = decltype(j_c)::value;
-    if (J < it.n_tiles) dma.template tile<J>(it.kv, J * TN);
+    if (J < it.n_tiles) dma.template tile<J>(it.kv, key_of(it, J));
   };
 
   Item cur;
@@ -1274,12 +1297,19 @@ dense_short_kernel(const PrefillParams p) {
   i32x4 kf[KR];
 
   auto mask_half = [&](int hh, f32x16& Sx) __attribute__((always_inline)) {
-    const int k0h = hh * 32;
-    if ((k0h + 32 > len) || (causal && k0h + 31 > q0w)) {
+    const int k0h = WIN ? key_of(cur, hh) : hh * 32;
+    bool edge = (k0h + 32 > len) || (causal && k0h + 31 > q0w);
+    // WIN: some key of the tile may lie below the local window of some row of the wave and outside the global one
+    if (WIN) edge = edge || (k0h <= q0w + 31 - wl && k0h + 31 >= wg);
+    if (edge) {
       const int t = row_lim - k0h - 8 * fr.lh;
+      const int below = t - wl;               // WIN: offsets up to here are at or below query - win_local ...
+      const int sink = wg - k0h - 8 * fr.lh;  // ... and are masked unless they are below this one (inside the global window)
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        if (16 * (r >> 3) + (r & 7) > t) Sx[r] = -INFINITY;
+      for (int r = 0; r < 16; ++r) {
+        const int kk = 16 * (r >> 3) + (r & 7);
+        if (kk > t || (WIN && kk <= below && kk >= sink)) Sx[r] = -INFINITY;
+      }
     }
   };
 
@@ -1371,7 +1401,7 @@ dense_short_kernel(const PrefillParams p) {
       __builtin_amdgcn_sched_barrier(0);
     }
     asm volatile("" : "+v"(Pc[4]), "+v"(Pc[5]), "+v"(Pc[6]), "+v"(Pc[7]), "+v"(rsv[KB]));
-    if (__builtin_amdgcn_ballot_w64(!(rsv[KB] <= kRowSumLimit)) != 0) exact_fix(Sc, Pc, rsv[KB]);
+    if (__builtin_amdgcn_ballot_w64(!(rsv[KB] <= kRowSumLimit) || (WIN && m == -INFINITY)) != 0) exact_fix(Sc, Pc, rsv[KB]);
     l += rsv[KB];
     mask_half(h + 1, Sn);
     __builtin_amdgcn_s_setprio(1);
@@ -1398,7 +1428,7 @@ dense_short_kernel(const PrefillParams p) {
       // tiles up to h+2 landed (requested at least two positions ago); tile h+3 may still fly
       __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 4) * 2 * IPW));
       __syncthreads();
-      dma.template tile<(J + NS - 1) % NS>(cur.kv, (h + NS - 1) * TN);
+      dma.template tile<(J + NS - 1) % NS>(cur.kv, key_of(cur, h + NS - 1));
     } else if (h == tail_h) {
       // nothing left to request: one full wait and one barrier publish what is
       // still on its way, and the waves run to the end of the item on their own
@@ -1476,6 +1506,7 @@ dense_short_kernel(const PrefillParams p) {
     row_lim = causal ? min(qrow, len - 1) : len - 1;
     H_w = (len + 31) / 32;
     if (causal) H_w = min(H_w, q0w / 32 + 1);
+    if (WIN) H_w -= cur.skip;  // (positions, not keys: the diagonal lies in the band)
     H_w = min(H_w, n_tiles);
     if (q0w >= len) H_w = 0;
     tail_h = max(1, n_tiles - (NS - 1));
@@ -1496,7 +1527,7 @@ dense_short_kernel(const PrefillParams p) {
 #pragma unroll
     for (int c = 0; c < G::KSTEPS; ++c) asm volatile("" : "+v"(Qf[c]));
     __syncthreads();
-    if (NS - 1 < n_tiles) dma.template tile<NS - 1>(cur.kv, (NS - 1) * TN);
+    if (NS - 1 < n_tiles) dma.template tile<NS - 1>(cur.kv, key_of(cur, NS - 1));
     if (H_w > 0) {
       f32x16 acc = (f32x16){0};
 #pragma unroll
@@ -1601,9 +1632,9 @@ inline bool short_form_pays(long long n128, long long n256, int cus) {
   return short_form_cost(n128, cus) < 2.3 * (double)((n256 + cus - 1) / cus);
 }
 
-template <typename T, int D>
+template <typename T, int D, bool WIN = false>
 int launch_short(const PrefillParams& p, long long items, int cus, hipStream_t s) {
-  auto kern = dense_short_kernel<T, D>;
+  auto kern = dense_short_kernel<T, D, WIN>;
   constexpr size_t lds = prefill_lds_bytes<D, kShortRows / 32, kShortStages, kShortTileKeys>();
   constexpr int per_cu = short_per_cu(D);
   static_assert(per_cu * lds <= 160 * 1024, "that many workgroups share a CU's LDS");
@@ -1657,6 +1688,13 @@ int launch_one(const PrefillParams& p, hipStream_t s) {
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), lds, s, pp);
   return (int)hipGetLastError();
+}
+
+// The token-window form without block lists: the 128-row form of the dense walk over each item's sink tiles and band.
+template <typename T, int D>
+int launch_window(const PrefillParams& p, hipStream_t s) {
+  const long long n = (long long)((p.max_seqlen + kShortRows - 1) / kShortRows) * p.hq * p.batch;
+  return launch_short<T, D, true>(p, n, device_cu_count(), s);
 }
 
 template <bool SPARSE>
@@ -1736,6 +1774,22 @@ int launch_prefill_dense(const PrefillParams& p, int dtype, int head_dim, hipStr
 }
 int launch_prefill_sparse(const PrefillParams& p, int dtype, int head_dim, hipStream_t s) {
   return dispatch<true>(p, dtype, head_dim, s);
+}
+int launch_prefill_window(const PrefillParams& p, int dtype, int head_dim, hipStream_t s) {
+  if (dtype == 0) {
+    switch (head_dim) {
+      case 64: return launch_window<__bf16, 64>(p, s);
+      case 96: return launch_window<__bf16, 96>(p, s);
+      case 128: return launch_window<__bf16, 128>(p, s);
+    }
+  } else {
+    switch (head_dim) {
+      case 64: return launch_window<_Float16, 64>(p, s);
+      case 96: return launch_window<_Float16, 96>(p, s);
+      case 128: return launch_window<_Float16, 128>(p, s);
+    }
+  }
+  return (int)hipErrorInvalidValue;
 }
 
 }  // namespace mi

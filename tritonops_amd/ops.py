@@ -17,6 +17,15 @@ from . import _lib
 from . import masks as _masks
 
 LOG2E = 1.4426950408889634
+# flash_attn_sparse_triton's window form runs either on block lists built on the
+# host (the block-list kernel, as every other mask) or without lists: the library
+# then walks each 128-row item's sink tiles and band with the dense kernel's
+# pipeline.  The second is 5 to 9 % faster for local windows of 2048 tokens or more
+# at head_dim 96 / 128 (B1 H16 S32768: 0.586 against 0.615 ms at 2048, 0.995 against
+# 1.087 ms at 4096) and up to 11 % slower for short windows and at head_dim 64, so
+# the choice is made per call.  True / False force one of the two (tests).
+WINDOW_PREFILL_LISTS = None
+_WINDOW_WALK_MIN_LOCAL = 2048
 _CU_COUNT = {}
 
 
@@ -460,10 +469,17 @@ def flash_attn_sparse_triton(q, k, v, cu_seqlens, softmax_scale=None, local_wind
             wl, wg = int(local_window_size), int(global_window_size)
             if wl < 0 or wg < 0:
                 raise ValueError("window sizes must be >= 0")
-            row_ptr, col_idx, csr_strides = _masks.window_csr(nqb, wl, wg, q.device)
+            # The library works the blocks out from the two windows when it
+            # gets no lists.  (local_window_size 0 hides even the diagonal; that
+            # case always goes through lists.)
+            use_lists = WINDOW_PREFILL_LISTS
+            if use_lists is None:
+                use_lists = not (D >= 96 and wl >= _WINDOW_WALK_MIN_LOCAL)
+            if wl < 1 or use_lists:
+                row_ptr, col_idx, csr_strides = _masks.window_csr(nqb, wl, wg, q.device)
         else:
             row_ptr, col_idx, csr_strides = _masks.block_mask_to_csr(block_mask, q.device)
-        if row_ptr.shape[-1] - 1 < nqb:
+        if row_ptr is not None and row_ptr.shape[-1] - 1 < nqb:
             raise ValueError("block mask covers %d query blocks, sequences need %d" % (row_ptr.shape[-1] - 1, nqb))
     if q.numel() == 0:
         return o, lse
