@@ -18,7 +18,7 @@ def _inputs(B, maxlen, Hq, Hkv, D, dtype=torch.bfloat16, lo=1):
 
 # (4, 2048, 4, 96) with LW=128, GW=0 is the reference's (disabled) test,
 # flash_attn_triton/flash_attn_sparse_attn_triton.py:445-503
-@pytest.mark.parametrize("lw,gw", [(128, 0), (128, 256), (100, 70), (1, 0), (64, 64), (5000, 0), (0, 5000), (0, 64)])
+@pytest.mark.parametrize("lw,gw", [(128, 0), (128, 256), (100, 70), (1, 0), (64, 64), (5000, 0), (0, 5000), (0, 64), (2 ** 40, 2 ** 40)])
 def test_window_sparse_matches_oracle(lw, gw):
     import tritonops_amd as ta
 

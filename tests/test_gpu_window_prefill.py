@@ -49,7 +49,7 @@ def _check(q, k, v, cu, lw, gw, tol=TOL):
 # windows shorter than a tile, ending inside tiles, longer than every sequence; no global
 # window (rows whose first tiles hold no visible key), a global window that meets the band
 @pytest.mark.parametrize("lw,gw", [(128, 0), (128, 256), (100, 70), (1, 0), (17, 0), (64, 64), (300, 0), (129, 65),
-                                   (5000, 0), (64, 5000), (1, 5000)])
+                                   (5000, 0), (64, 5000), (1, 5000), (2 ** 40, 2 ** 40)])
 @pytest.mark.parametrize("D,dtype", [(96, torch.bfloat16), (128, torch.bfloat16), (64, torch.float16)])
 def test_window_walk_matches_oracle(no_lists, lw, gw, D, dtype):
     import tritonops_amd as ta

@@ -2,6 +2,7 @@
 // Nothing in this file touches the device except the final kernel launches.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -500,7 +501,8 @@ int mi_attn_fwd_blocksparse(const mi_attn_sparse_args* a, void* stream) {
   p.row_ptr = a->row_ptr; p.col_idx = a->col_idx;
   p.rp_sb = a->row_ptr_stride_b; p.rp_sh = a->row_ptr_stride_h;
   p.ci_sb = a->col_idx_stride_b; p.ci_sh = a->col_idx_stride_h;
-  p.win_local = a->window_local; p.win_global = a->window_global;
+  // (-1 stays -1; a window as long as the longest sequence already is the whole sequence)
+  p.win_local = std::min(a->window_local, a->max_seqlen); p.win_global = std::min(a->window_global, a->max_seqlen);
   return launch_status(mi::launch_prefill_sparse(p, a->dtype, a->head_dim, static_cast<hipStream_t>(stream)), "mi_attn_fwd_blocksparse");
 }
 

@@ -469,6 +469,7 @@ def flash_attn_sparse_triton(q, k, v, cu_seqlens, softmax_scale=None, local_wind
             wl, wg = int(local_window_size), int(global_window_size)
             if wl < 0 or wg < 0:
                 raise ValueError("window sizes must be >= 0")
+            wl, wg = min(wl, 2 ** 31 - 1), min(wg, 2 ** 31 - 1)   # (the C ABI takes 32-bit windows; longer than any sequence either way)
             # The library works the blocks out from the two windows when it
             # gets no lists.  (local_window_size 0 hides even the diagonal; that
             # case always goes through lists.)
