@@ -56,6 +56,7 @@ KERNELS = {
 KERNELS["dense_causal_packed"] = KERNELS["dense_causal"]
 KERNELS["window_sparse_prefill"] = KERNELS["block_sparse"]
 KERNELS["window_sparse_decode"] = KERNELS["sparse_decode"]
+KERNELS["window_long_prefill"] = _NS + "18dense_short_kernelIDF16bLi128ELb1EEEvNS_13PrefillParamsE"   # the dense walk over a window's tiles
 
 
 def _sync():
@@ -678,18 +679,17 @@ def _window_pairs(n, lw, gw):
     return int((np.minimum(qi + 1, lw) + np.maximum(0, np.minimum(gw, qi + 1 - lw))).sum())
 
 
-def run_window_sparse_prefill(steps, warmup):
-    """The reference's own sparse prefill form: token windows on packed tensors
-    (flash_attn_sparse_attn_triton.py:237-326), local window 1024, global window 128, 4 sequences of 8192 tokens."""
+def _run_window_prefill(name, B, H, S, LW, GW, lists, steps, warmup):
+    """flash_attn_sparse_triton(q, k, v, cu, None, LW, GW) on B packed sequences of S tokens, head_dim 128; the
+    device-time leg goes through the C ABI with the window's block lists (`lists`) or without any."""
     import tritonops_amd as ta
     from tritonops_amd import _lib, masks
-    B, H, S, D, LW, GW = 4, 16, 8192, 128, 1024, 128
+    D = 128
     T = B * S
     q, k, v = (_randn((1, T, H, D), s) for s in (0, 1, 2))
     cu = (torch.arange(B + 1, dtype=torch.int32) * S).cuda()
     fn = lambda: ta.flash_attn_sparse_triton(q, k, v, cu, None, LW, GW)
     o, lse = fn()
-    row_ptr, col_idx, strides = masks.window_csr(S // 64, LW, GW, "cuda")
     o2, lse2 = torch.empty_like(o), torch.empty_like(lse)
     a = _lib.AttnSparseArgs()
     a.struct_size = C.sizeof(a)
@@ -700,8 +700,10 @@ def run_window_sparse_prefill(steps, warmup):
         setattr(a, n + "_stride_h", t.stride(2))
     a.lse_stride_s, a.lse_stride_h = lse2.stride(1), lse2.stride(2)
     a.cu_seqlens = cu.data_ptr()
-    a.row_ptr, a.col_idx = row_ptr.data_ptr(), col_idx.data_ptr()
-    a.row_ptr_stride_b, a.row_ptr_stride_h, a.col_idx_stride_b, a.col_idx_stride_h = strides
+    if lists:
+        row_ptr, col_idx, strides = masks.window_csr(S // 64, LW, GW, "cuda")
+        a.row_ptr, a.col_idx = row_ptr.data_ptr(), col_idx.data_ptr()
+        a.row_ptr_stride_b, a.row_ptr_stride_h, a.col_idx_stride_b, a.col_idx_stride_h = strides
     a.batch, a.heads_q, a.heads_kv, a.max_seqlen, a.head_dim = B, H, H, S, D
     a.block_size, a.window_local, a.window_global = 64, LW, GW
     a.scale_log2 = D ** -0.5 * LOG2E
@@ -711,7 +713,7 @@ def run_window_sparse_prefill(steps, warmup):
     flop = 4.0 * D * _window_pairs(S, LW, GW) * H * B
     err = err_lse = 0.0
     keys = torch.arange(S, device="cuda")
-    for b in (0, 3):
+    for b in sorted({0, B - 1}):
         for r0 in (0, 1024, 4160, S - 64):
             rows = torch.arange(r0, r0 + 64, device="cuda")
             allow = (keys[None, :] <= rows[:, None]) & ((rows[:, None] - keys[None, :] < LW) | (keys[None, :] < GW))
@@ -721,17 +723,33 @@ def run_window_sparse_prefill(steps, warmup):
             err = max(err, _err(o[0, b * S + rows].transpose(0, 1), want))
             err_lse = max(err_lse, _err(lse[0, b * S + rows].transpose(0, 1), want_lse))
     return {
-        "name": "window_sparse_prefill", "ms_per_step": ms, "kernel_ms": kms,
+        "name": name, "ms_per_step": ms, "kernel_ms": kms,
         "metric": "sparse_attn_fwd_tflops", "unit": "TFLOP/s", "value": flop / (ms * 1e-3) / 1e12,
         "max_abs_err": err, "max_abs_err_lse2": err_lse,
-        "err_sample": "o and lse of all heads x 4 blocks of 64 query rows in 2 of the 4 sequences against masked fp32 torch math on the device",
+        "err_sample": "o and lse of all heads x 4 blocks of 64 query rows in %d of the %d sequences against masked fp32 torch "
+                      "math on the device" % (len({0, B - 1}), B),
         "roofline": {"bound": "mfma", "achieved": flop / (kms * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "kernel": KERNELS["window_sparse_prefill"]},
-        "config": {"workload": "window-sparse causal fwd bf16, packed [1,32768,16,128] + cu_seqlens for 4 x 8192 tokens, local "
-                               "window 1024, global window 128, through flash_attn_sparse_triton(q, k, v, cu, None, 1024, 128)",
+                     "unit": "TFLOP/s", "kernel": KERNELS[name]},
+        "config": {"workload": "window-sparse causal fwd bf16, packed [1,%d,%d,128] + cu_seqlens for %d x %d tokens, local "
+                               "window %d, global window %d, through flash_attn_sparse_triton(q, k, v, cu, None, %d, %d)"
+                               % (T, H, B, S, LW, GW, LW, GW),
                    "flop_per_step": flop, "wall_over_kernel": ms / kms,
-                   "note": "FLOP counts the allowed (q, k) pairs only; the kernel walks whole 64x64 blocks that hold one"},
+                   "note": ("FLOP counts the allowed (q, k) pairs only; the kernel walks whole 64x64 blocks that hold one" if lists else
+                            "FLOP counts the allowed (q, k) pairs only; no block lists: the library walks each 128-row item's "
+                            "sink tiles and band (whole 32-key tiles)")},
     }
+
+
+def run_window_sparse_prefill(steps, warmup):
+    """The reference's own sparse prefill form: token windows on packed tensors
+    (flash_attn_sparse_attn_triton.py:237-326), local window 1024, global window 128, 4 sequences of 8192 tokens."""
+    return _run_window_prefill("window_sparse_prefill", 4, 16, 8192, 1024, 128, True, steps, warmup)
+
+
+def run_window_long_prefill(steps, warmup):
+    """The same call form with a long local window on a long sequence (4096 / 128, one sequence of 32768 tokens):
+    the case the drop-in sends to the library without block lists."""
+    return _run_window_prefill("window_long_prefill", 1, 16, 32768, 4096, 128, False, steps, warmup)
 
 
 def run_window_sparse_decode(steps, warmup):
@@ -812,6 +830,7 @@ WORKLOADS = {
     "dense_causal_packed": run_dense_packed,
     "window_sparse_prefill": run_window_sparse_prefill,
     "window_sparse_decode": run_window_sparse_decode,
+    "window_long_prefill": run_window_long_prefill,
 }
 
 # Parity bars: the largest error a workload's own check may report (its figure under "max_abs_err",
@@ -829,6 +848,7 @@ PARITY_BARS = {
     "dense_causal_packed": {"max_abs_err": 2e-2, "max_abs_err_lse2": 2e-3},
     "window_sparse_prefill": {"max_abs_err": 2e-2, "max_abs_err_lse2": 2e-3},
     "window_sparse_decode": {"max_abs_err": 2e-2},
+    "window_long_prefill": {"max_abs_err": 2e-2, "max_abs_err_lse2": 2e-3},
 }
 
 
@@ -964,6 +984,18 @@ def cpu_baseline(name):
                 "sample": "torch-CPU window oracle (flash_attn_sparse_attn_triton.py:391-442: full S x S scores, then the "
                           "mask) on one sequence of 8192 tokens, 4 of the 16 heads (1/16 of the workload), one timed run "
                           "after a warm-up; same algorithmic-FLOP formula as the GPU figure (allowed pairs only)",
+                "seconds": t}
+    if name == "window_long_prefill":
+        S, H, D, LW, GW = 8192, 4, 128, 4096, 128
+        q, k, v = (torch.randn((1, S, H, D), generator=g).to(torch.bfloat16) for _ in range(3))
+        cu = torch.tensor([0, S], dtype=torch.int32)
+        t = med(lambda: orc.flash_attn_sparse_torch(q, k, v, cu, None, LW, GW), reps=1)
+        flop = 4.0 * D * _window_pairs(S, LW, GW) * H
+        return {"value": flop / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "sample": "torch-CPU window oracle (flash_attn_sparse_attn_triton.py:391-442: full S x S scores, then the "
+                          "mask) with the same two windows on a sequence of 8192 tokens (a quarter of the workload's) and 4 "
+                          "of the 16 heads, one timed run after a warm-up; same algorithmic-FLOP formula as the GPU figure "
+                          "(allowed pairs only)",
                 "seconds": t}
     if name == "window_sparse_decode":
         B, Hq, Hkv, L, D, GW, LW = 1, 32, 8, 131072, 128, 256, 4096
