@@ -23,6 +23,9 @@
 //     path): equals the plain softmax, also for scores that keep growing.
 //   decode (decode.hip): the window form's arithmetic block list equals the
 //     set of blocks that hold an attended token; live chunks are dealt once.
+//   window walk (prefill.hip, dense_short_kernel with WIN): the tiles an item
+//     of the two-window form walks, the positions each wave works on and the
+//     tile masks let every query see exactly the keys the window rule allows.
 #include <algorithm>
 #include <cassert>
 #include <cmath>
@@ -759,6 +762,97 @@ static void test(std::mt19937& rng) {
 }
 }  // namespace decode
 
+// ------------------------------------------------------- window walk (prefill)
+// dense_short_kernel<T, D, WIN = true>: a 128-row item of the two-window form
+// walks the tiles (32 keys) of the first win_global keys, then the band that
+// ends at its diagonal block.  Restated here: the item's walk (next_item), the
+// key of a position (key_of), the positions a wave works on (H_w) and the mask
+// of a tile (mask_half).  Checked against the rule itself - key k is visible to
+// query r iff k <= r and (r - k < wl or k < wg) - for every row of every wave.
+namespace window_walk {
+constexpr int TN = 32, BM = 128, NW = 4;
+struct Walk {
+  int n_sink, skip, n_tiles;
+  int key_of(int j) const { return (j + (j >= n_sink ? skip : 0)) * TN; }
+};
+static Walk item_walk(int q0, int len, int wl, int wg) {
+  Walk w;
+  w.n_tiles = std::min((len + TN - 1) / TN, (q0 + BM + TN - 1) / TN);  // causal
+  const int t0 = std::max(q0 - wl + 1, 0) / TN;
+  w.n_sink = g_mut == 14 ? (wg + TN - 1) / TN : std::min((wg + TN - 1) / TN, t0);
+  w.skip = t0 - w.n_sink;
+  w.n_tiles -= w.skip;
+  return w;
+}
+static int wave_positions(const Walk& w, int q0w, int len) {
+  int h = std::min((len + 31) / 32, q0w / 32 + 1);
+  if (g_mut != 13) h -= w.skip;
+  h = std::min(h, w.n_tiles);
+  return q0w >= len ? 0 : h;
+}
+// is key k0h + off masked for the lane whose query is `row` (already cut at len - 1)?
+static bool masked(int k0h, int off, int row, int q0w, int len, int wl, int wg, bool& edge) {
+  edge = (k0h + 32 > len) || (k0h + 31 > q0w);
+  if (g_mut != 15) edge = edge || (k0h <= q0w + 31 - wl && k0h + 31 >= wg);
+  if (!edge) return false;
+  const int t = row - k0h;
+  const int below = t - wl, sink = wg - k0h;
+  return off > t || (off <= below && off >= sink);
+}
+
+static void test(std::mt19937& rng) {
+  int cases = 0;
+  for (int rep = 0; rep < 6000; ++rep) {
+    const int len = rep < 300 ? 1 + rep : 1 + (int)(rng() % 5000);
+    const int wl = rep % 7 == 0 ? 1 + (int)(rng() % 40) : 1 + (int)(rng() % 3000);
+    const int wg = rep % 3 == 0 ? 0 : (int)(rng() % 400);
+    const int n_items = (len + BM - 1) / BM;
+    const int item = (int)(rng() % n_items), q0 = item * BM;
+    const Walk w = item_walk(q0, len, wl, wg);
+    CHECK(w.n_tiles >= 1, "item at row %d walks %d tiles (len %d, wl %d, wg %d)", q0, w.n_tiles, len, wl, wg);
+    int prev = -1;
+    for (int j = 0; j < w.n_tiles; ++j) {
+      const int k0 = w.key_of(j);
+      CHECK(k0 > prev && k0 < len, "position %d is tile %d after tile %d (len %d, q0 %d, wl %d, wg %d)", j, k0 / TN, prev / TN, len, q0, wl, wg);
+      prev = k0;
+    }
+    for (int wave = 0; wave < NW; ++wave) {
+      const int q0w = q0 + 32 * wave;
+      const int H = wave_positions(w, q0w, len);
+      CHECK(H >= 0 && H <= w.n_tiles, "wave %d works on %d of %d positions", wave, H, w.n_tiles);
+      if (q0w >= len) continue;
+      // no position that lies wholly above the wave's diagonal is worked on
+      CHECK(H >= 1 && w.key_of(H - 1) <= std::min(q0w + 31, len - 1), "wave %d works on %d positions, the last one from key %d on, above its rows %d.. (skip %d)",
+            wave, H, H >= 1 ? w.key_of(H - 1) : -1, q0w, w.skip);
+      for (int lq = 0; lq < 32; ++lq) {
+        const int row = std::min(q0w + lq, len - 1);   // rows past the end repeat the last one
+        // what the walk lets this row see
+        std::vector<char> seen(len, 0);
+        for (int j = 0; j < H; ++j) {
+          const int k0h = w.key_of(j);
+          for (int off = 0; off < 32; ++off) {
+            bool edge;
+            const bool m = masked(k0h, off, row, q0w, len, wl, wg, edge);
+            if (!m) {
+              CHECK(k0h + off < len, "row %d sees key %d of a sequence of %d tokens", row, k0h + off, len);
+              if (k0h + off < len) seen[k0h + off] = 1;
+            }
+          }
+        }
+        for (int k = 0; k < len; ++k) {
+          const bool want = k <= row && (row - k < wl || k < wg);
+          CHECK((bool)seen[k] == want, "row %d %s key %d (len %d, q0 %d, wave %d, wl %d, wg %d, sink %d skip %d tiles %d H %d)",
+                row, want ? "misses" : "wrongly sees", k, len, q0, wave, wl, wg, w.n_sink, w.skip, w.n_tiles, H);
+          if ((bool)seen[k] != want) break;
+        }
+      }
+    }
+    ++cases;
+  }
+  std::printf("window walk: %d items\n", cases);
+}
+}  // namespace window_walk
+
 int main(int argc, char** argv) {
   if (argc > 1) g_mut = std::atoi(argv[1]);
   std::mt19937 rng(12345);
@@ -766,6 +860,7 @@ int main(int argc, char** argv) {
   sparse::test(rng);
   softmax::test(rng);
   decode::test(rng);
+  window_walk::test(rng);
   if (g_fail) {
     std::printf("%d check(s) failed\n", g_fail);
     return 1;

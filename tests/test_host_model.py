@@ -30,6 +30,9 @@ MISTAKES = {
     10: "block-sparse: the list register behind the walked one is refilled with the wrong 64 entries",
     11: "short form: the wait at the top of an item always leaves one tile in flight",
     12: "short form: the wait at the top of a position leaves two tiles in flight",
+    13: "window walk: a wave's positions are counted in keys, not in positions of the walk",
+    14: "window walk: the sink tiles are not cut at the first tile of the band",
+    15: "window walk: a tile at the window's lower edge is taken for unmasked",
 }
 
 
@@ -54,7 +57,7 @@ def test_walks_hold_their_invariants(model):
     r = _run(model)
     assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
     assert "host model ok" in r.stdout
-    for part in ("dense walk", "block-sparse walk", "softmax reference point", "decode lists and chunks"):
+    for part in ("dense walk", "block-sparse walk", "softmax reference point", "decode lists and chunks", "window walk"):
         assert part in r.stdout
 
 
