@@ -68,15 +68,19 @@ def test_block_sparse_prefill_random_masks(seed):
 WINDOW_LENGTHS = [1, 31, 33, 64, 65, 127, 128, 192, 200, 257, 320, 384, 513, 700, 1000]
 
 
+@pytest.mark.parametrize("lists", [True, False], ids=["lists", "no-lists"])
 @pytest.mark.parametrize("seed", range(8))
-def test_window_sparse_prefill_random_windows(seed):
+def test_window_sparse_prefill_random_windows(seed, lists, monkeypatch):
     """Ragged batches through the window form with windows small enough that a
     row's first listed tile can lie wholly outside its window (the row then has
     no reference point for its probabilities yet) and with large scores (the
     reference point has to move).  Output and LSE against the oracle; rows
-    without any visible key must come back as o = 0, lse = -inf."""
+    without any visible key must come back as o = 0, lse = -inf.  Both ways the
+    drop-in can run the form: block lists built on the host, and no lists."""
     import tritonops_amd as ta
+    from tritonops_amd import ops
 
+    monkeypatch.setattr(ops, "WINDOW_PREFILL_LISTS", lists)
     rnd = random.Random(200 + seed)
     lens = [rnd.choice(WINDOW_LENGTHS) for _ in range(rnd.randint(1, 4))]
     Hkv = rnd.choice([1, 2, 4])
