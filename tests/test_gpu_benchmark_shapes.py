@@ -1,7 +1,7 @@
 """GPU parity at the full benchmark shapes that the other test files reach only
 in reduced form: block-sparse prefill at B2 H16 S16384, block-list decoding at
-B32 Hkv8 KV131072 with 128 listed blocks + the last one, and the dense backward
-at B4 H32 S8192.  Inputs of these sizes are drawn on the device; the checks
+B32 Hkv8 KV131072 with 128 listed blocks + the last one, the dense backward
+at B4 H32 S8192, and the window prefill without block lists on 32768 tokens.  Inputs of these sizes are drawn on the device; the checks
 are the CPU oracle on slices that it finishes in seconds, fp32 torch math on
 the device for sampled heads, and size-independent properties."""
 import pytest
@@ -130,3 +130,42 @@ def test_dense_backward_at_the_benchmark_shape():
     _, _, dv1 = ops._dense_bwd(qs, ks, vs, o, ds1, lse, None, sm, True, None)
     col = dv1.float().mean(-1)                                     # [B, S, H]: every column of dv[j] equals sum_i P[i, j]
     assert (col.sum(1) - S).abs().max().item() <= 1e-3 * S
+
+
+def test_window_prefill_without_lists_at_the_benchmark_shape():
+    """One packed sequence of 32768 tokens, 16 heads, local window 4096 / global 128 (bench.py's
+    window_long_prefill), through the call without block lists: sampled blocks of query rows of every
+    head against masked fp32 math on the device, the same call through the window's block lists, and
+    the size-independent property that a local window as long as the sequence is dense causal attention."""
+    import tritonops_amd as ta
+    from tritonops_amd import ops
+
+    S, H, D, LW, GW = 32768, 16, 128, 4096, 128
+    q, k, v = (_randn_dev((1, S, H, D), s) for s in (11, 12, 13))
+    cu = torch.tensor([0, S], dtype=torch.int32, device="cuda")
+    assert ops.WINDOW_PREFILL_LISTS is None            # the drop-in's own choice: no lists at this window
+    o, lse = ta.flash_attn_sparse_triton(q, k, v, cu, None, LW, GW)
+    keys = torch.arange(S, device="cuda")
+    qh, kh, vh = (t[0].transpose(0, 1).float() for t in (q, k, v))      # [H, S, D]
+    for r0 in (0, 64, 4032, 4096, 4160, 20000, S - 64):
+        rows = torch.arange(r0, r0 + 64, device="cuda")
+        allow = (keys[None, :] <= rows[:, None]) & ((rows[:, None] - keys[None, :] < LW) | (keys[None, :] < GW))
+        s = torch.einsum("hqd,hkd->hqk", qh[:, rows], kh) * D ** -0.5
+        s = s.masked_fill(~allow[None], float("-inf"))
+        want = torch.einsum("hqk,hkd->hqd", torch.softmax(s, -1), vh)
+        assert_close(o[0, rows].transpose(0, 1), want, TOL)
+        assert (lse[0, rows].transpose(0, 1) - torch.logsumexp(s, -1) * orc.LOG2E).abs().max().item() <= LSE_TOL
+    old = ops.WINDOW_PREFILL_LISTS
+    try:
+        ops.WINDOW_PREFILL_LISTS = True
+        o_l, lse_l = ta.flash_attn_sparse_triton(q, k, v, cu, None, LW, GW)
+        assert_close(o, o_l, 1e-2)                     # two kernels, two summation orders
+        assert (lse - lse_l).abs().max().item() <= LSE_TOL
+        del o_l, lse_l
+        ops.WINDOW_PREFILL_LISTS = False
+        o_full, lse_full = ta.flash_attn_sparse_triton(q, k, v, cu, None, S, 0)
+    finally:
+        ops.WINDOW_PREFILL_LISTS = old
+    o_dense, lse_dense = ta.flash_attn_triton_fwd(q, k, v, cu, D ** -0.5 * orc.LOG2E)
+    assert_close(o_full, o_dense, 1e-2)
+    assert (lse_full - lse_dense).abs().max().item() <= LSE_TOL
