@@ -105,3 +105,59 @@ def test_packed_forward_and_backward_replay_like_eager():
         torch.cuda.synchronize()
         for g, w in zip(got, want):
             assert torch.equal(g, w), rep
+
+
+def test_sparse_prefill_forms_replay_like_eager():
+    """The sparse prefill under capture: a block mask through a prebuilt CSR, and the two-window form both
+    ways the drop-in can run it (block lists, which are built once per window pair and kept on the host
+    side, and no lists at all).  Packed tensors with rows that belong to no sequence, so the launch that
+    zeroes them is part of the graph as well."""
+    import tritonops_amd as ta
+    from tritonops_amd import masks, ops
+
+    Hq, Hkv, D, lw, gw = 4, 2, 128, 300, 70
+    lens = [700, 0, 333]
+    T = sum(lens) + 40                                  # 40 rows behind the last sequence
+    cu = torch.tensor([0, 700, 700, 1033], device="cuda", dtype=torch.int32)
+    q = torch.empty((1, T, Hq, D), device="cuda", dtype=torch.bfloat16)
+    k = torch.empty((1, T, Hkv, D), device="cuda", dtype=torch.bfloat16)
+    v = torch.empty_like(k)
+    inputs = (q, k, v)
+    csr = masks.block_mask_to_csr(masks.synthetic_block_mask(11, band=2, sink=1, frac=0.3, seed=5), "cuda")
+
+    def run():
+        out = []
+        old = ops.WINDOW_PREFILL_LISTS
+        try:
+            for lists in (True, False):
+                ops.WINDOW_PREFILL_LISTS = lists
+                out += ta.flash_attn_sparse_triton(q, k, v, cu, None, lw, gw, max_seq_len=700)
+        finally:
+            ops.WINDOW_PREFILL_LISTS = old
+        out += ta.flash_attn_sparse_triton(q, k, v, cu, row_ptr=csr[0], col_idx=csr[1], csr_strides=csr[2], max_seq_len=700)
+        return out
+
+    for i, t in enumerate(inputs):
+        _fill(t, 300 + i)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()                                  # loads the library, sets kernel attributes, builds the window's lists
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        captured = run()
+    for rep in range(3):
+        for i, t in enumerate(inputs):
+            _fill(t, 3000 * (rep + 1) + i)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        want = run()
+        torch.cuda.synchronize()
+        for g, w in zip(got, want):
+            assert torch.equal(g, w), rep
+        assert torch.count_nonzero(got[0][0, 1033:]) == 0 and torch.count_nonzero(got[2][0, 1033:]) == 0
