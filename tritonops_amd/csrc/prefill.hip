@@ -9,7 +9,9 @@
 // items and requests the first tiles of its next item while it writes out the
 // current one, and a software pipeline over half tiles inside each wavefront
 // (see dense_kernel).  Block-sparse: the same pipeline over 32-key tiles of
-// the listed blocks, two stages per tensor, one launch per item.
+// the listed blocks, two stages per tensor, one launch per item.  The sparse
+// launcher's two-window form also runs without lists: the 128-row form of the
+// dense walk over each item's sink tiles and band (dense_short_kernel, WIN).
 //
 // Replaces flash_attn_fwd_kernel of flash_attn_triton/flash_attn_triton.py
 // :52-180 (dense) and flash_attn_triton/flash_attn_sparse_attn_triton.py
